@@ -51,10 +51,27 @@ int dgi_ssm_scan(float* y, const float* xbc, int xbc_stride, const void* dt_raw,
 int dgi_gated_group_norm(void* out, int out_f32, const float* y, const void* z, int z_f32, int z_stride, const float* w,
                          int T, int C, int groups, float eps, hipStream_t s);
 int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const float* corr, int T, int R, int top,
-                  hipStream_t s);
+                  int sigmoid, hipStream_t s);
+int dgi_glu_rows(void* out, const void* gu, int gu_stride, int rows, int I, int kind, float limit, float alpha,
+                 const float* row_scale, int is_f32, hipStream_t s);
+int dgi_stream_add_norm(float* x, int T, int W, const void* y, int y_stride, int y_f32, const float* post_w,
+                        const float* next_w, float eps, void* out, int out_f32, hipStream_t s);
+int dgi_latent_prep(const void* proj, int stride, int is_f32, int T, int q_rank, int kv_rank, int rot_dim,
+                    const float* dq_w, const float* dkv_w, float eps, const int* positions, const int* slots,
+                    const float* cos_sin, int dims, int interleaved, void* cq, void* cache, hipStream_t s);
+int dgi_gate_heads(void* out, const void* ov, long long ov_hs, long long ov_ts, const void* gate, int gate_stride,
+                   int per_head, int T, int H, int dv, int is_f32, hipStream_t s);
+int dgi_gelu_tanh(void* out, const void* x, int x_stride, int rows, int n, const void* table, int t_stride, int vocab,
+                  const int* ids, int col0, int is_f32, hipStream_t s);
+int dgi_latent_attn_rows(const void* q, int q_stride, const void* q_lat, long long ql_hs, long long ql_ts,
+                         const void* cache, const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs,
+                         const int* positions, int rows, int H, int dim, int rd, int kr, int block_size, float scale,
+                         int window, const float* cos_sin, int dims, int interleaved, void* out, long long o_hs,
+                         long long o_ts, int is_f32, hipStream_t s);
 int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s);
 int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up, int T, int E,
-                           int top, int ff, int W, int is_f32, hipStream_t s);
+                           int top, int ff, int W, const float* pair_scale, int act, float limit, float alpha, int is_f32,
+                           hipStream_t s);
 int dgi_moe_expert_down(void* ys, const float* mid, const int* idx, const void* down, int T, int E, int top, int ff, int W,
                         int is_f32, hipStream_t s);
 int dgi_moe_combine(void* out, const void* ys, const int* where, const void* h, int h_stride, const int* idx,
@@ -415,14 +432,14 @@ void gated_group_norm(at::Tensor out, const at::Tensor& y, const at::Tensor& z, 
            "gated_group_norm");
 }
 
-void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits, const at::Tensor& corr) {
+void moe_route(at::Tensor idx, at::Tensor wts, const at::Tensor& logits, const c10::optional<at::Tensor>& corr,
+               int64_t sigmoid) {
   check_i32(idx, "idx"); check_f32(wts, "wts");
   TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == at::kFloat && logits.dim() == 2 && logits.stride(1) == 1);
   const int T = (int)logits.size(0), R = (int)logits.size(1);
   TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes());
-  check_f32(corr, "correction", R);
   check_rc(dgi_moe_route(idx.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(), (int)logits.stride(0),
-                         corr.data_ptr<float>(), T, R, (int)idx.size(1), cur_stream()), "moe_route");
+                         f32p(corr, "correction", R), T, R, (int)idx.size(1), (int)sigmoid, cur_stream()), "moe_route");
 }
 
 void glu_silu(at::Tensor out, const at::Tensor& gu) {
@@ -435,14 +452,16 @@ void glu_silu(at::Tensor out, const at::Tensor& gu) {
 }
 
 // gate_up [E, 2 ff, W], down [E, W, ff] in h's dtype; idx [T, top]; mid [T * top, ff] fp32; ys [T * top, W]
-void moe_expert_gate_up(at::Tensor mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& gate_up) {
+void moe_expert_gate_up(at::Tensor mid, const at::Tensor& h, const at::Tensor& idx, const at::Tensor& gate_up,
+                        const c10::optional<at::Tensor>& pair_scale, int64_t act, double limit, double alpha) {
   const int f = act_kind(h, "h");
   check_rows(h, "h"); check_f32(mid, "mid"); check_i32(idx, "idx");
   TORCH_CHECK(act_kind(gate_up, "gate_up") == f && gate_up.is_contiguous() && gate_up.dim() == 3 && gate_up.size(2) == h.size(1));
   const int T = (int)h.size(0), W = (int)h.size(1), E = (int)gate_up.size(0), ff = (int)gate_up.size(1) / 2;
   TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && mid.numel() == (int64_t)T * idx.size(1) * ff);
   check_rc(dgi_moe_expert_gate_up(mid.data_ptr<float>(), h.data_ptr(), (int)h.stride(0), idx.data_ptr<int>(),
-                                  gate_up.data_ptr(), T, E, (int)idx.size(1), ff, W, f, cur_stream()), "moe_expert_gate_up");
+                                  gate_up.data_ptr(), T, E, (int)idx.size(1), ff, W, f32p(pair_scale, "pair_scale", idx.numel()),
+                                  (int)act, (float)limit, (float)alpha, f, cur_stream()), "moe_expert_gate_up");
 }
 
 void moe_expert_down(at::Tensor ys, const at::Tensor& mid, const at::Tensor& idx, const at::Tensor& down) {
@@ -457,9 +476,9 @@ void moe_expert_down(at::Tensor ys, const at::Tensor& mid, const at::Tensor& idx
 }
 
 void moe_combine(at::Tensor out, const at::Tensor& ys, const c10::optional<at::Tensor>& where, const at::Tensor& h, const at::Tensor& idx,
-                 const at::Tensor& wts, const c10::optional<at::Tensor>& shared, int64_t E) {
+                 const c10::optional<at::Tensor>& wts, const c10::optional<at::Tensor>& shared, int64_t E) {
   const int f = act_kind(h, "h");
-  check_rows(h, "h"); check_i32(idx, "idx"); check_f32(wts, "wts");
+  check_rows(h, "h"); check_i32(idx, "idx");
   const int* wp = nullptr;
   if (where.has_value()) {
     check_i32(*where, "where");
@@ -469,7 +488,7 @@ void moe_combine(at::Tensor out, const at::Tensor& ys, const c10::optional<at::T
   const int T = (int)h.size(0), W = (int)h.size(1);
   TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.size(0) == T && out.size(1) == W);
   TORCH_CHECK(act_kind(ys, "ys") == f && ys.is_contiguous() && ys.dim() == 2 && ys.size(1) == W);
-  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T && wts.sizes() == idx.sizes());
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T);
   TORCH_CHECK(where.has_value() || ys.size(0) == idx.numel(), "moe_combine: without `where` ys holds one row per pair");
   const void* sp = nullptr;
   int ss = 0;
@@ -479,8 +498,161 @@ void moe_combine(at::Tensor out, const at::Tensor& ys, const c10::optional<at::T
     sp = shared->data_ptr(); ss = (int)shared->stride(0);
   }
   check_rc(dgi_moe_combine(out.data_ptr(), ys.data_ptr(), wp, h.data_ptr(), (int)h.stride(0),
-                           idx.data_ptr<int>(), wts.data_ptr<float>(), sp, ss, T, (int)E, (int)idx.size(1), W, f, cur_stream()),
+                           idx.data_ptr<int>(), f32p(wts, "wts", idx.numel()), sp, ss, T, (int)E, (int)idx.size(1), W, f, cur_stream()),
            "moe_combine");
+}
+
+void glu_rows(at::Tensor out, const at::Tensor& gu, int64_t kind, double limit, double alpha,
+              const c10::optional<at::Tensor>& row_scale) {
+  const int f = act_kind(gu, "gu");
+  check_rows(gu, "gu");
+  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.dim() == 2 && out.size(0) == gu.size(0) &&
+              2 * out.size(1) == gu.size(1));
+  check_rc(dgi_glu_rows(out.data_ptr(), gu.data_ptr(), (int)gu.stride(0), (int)gu.size(0), (int)out.size(1), (int)kind,
+                        (float)limit, (float)alpha, f32p(row_scale, "row_scale", gu.size(0)), f, cur_stream()), "glu_rows");
+}
+
+// x [T, W] fp32 += y (unit-RMS normed and weighted if post_w); out = RMS norm of x times next_w (or x) in out's dtype
+void stream_add_norm(at::Tensor x, const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& post_w,
+                     const c10::optional<at::Tensor>& next_w, double eps, c10::optional<at::Tensor> out) {
+  check_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2);
+  const int T = (int)x.size(0), W = (int)x.size(1);
+  const void* yp = nullptr;
+  int ys = 0, yf = 1;
+  if (y.has_value()) {
+    yf = act_kind(*y, "y");
+    check_rows(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == W, "stream_add_norm: y must be [T, W]");
+    yp = y->data_ptr(); ys = (int)y->stride(0);
+  }
+  TORCH_CHECK(!post_w.has_value() || y.has_value(), "stream_add_norm: post_w needs y");
+  void* op = nullptr;
+  int of = 1;
+  if (out.has_value()) {
+    of = act_kind(*out, "out");
+    TORCH_CHECK(out->is_contiguous() && out->dim() == 2 && out->size(0) == T && out->size(1) == W);
+    op = out->data_ptr();
+  }
+  check_rc(dgi_stream_add_norm(x.data_ptr<float>(), T, W, yp, ys, yf, f32p(post_w, "post_w", W), f32p(next_w, "next_w", W),
+                               (float)eps, op, of, cur_stream()), "stream_add_norm");
+}
+
+void latent_prep(at::Tensor cq, const at::Tensor& proj, int64_t q_rank, int64_t kv_rank, int64_t rot_dim,
+                 const at::Tensor& dq_w, const c10::optional<at::Tensor>& dkv_w, double eps, const at::Tensor& positions,
+                 const at::Tensor& slots, const c10::optional<at::Tensor>& cos_sin, bool interleaved,
+                 c10::optional<at::Tensor> cache) {
+  const int f = act_kind(proj, "proj");
+  check_rows(proj, "proj");
+  const int T = (int)proj.size(0);
+  TORCH_CHECK(q_rank > 0 && kv_rank >= 0 && rot_dim >= 0 && proj.size(1) >= q_rank + kv_rank + rot_dim,
+              "latent_prep: proj rows are [q_rank | kv_rank | rot_dim | ...]");
+  TORCH_CHECK(act_kind(cq, "cq") == f && cq.is_contiguous() && cq.dim() == 2 && cq.size(0) == T && cq.size(1) == q_rank);
+  check_f32(dq_w, "dq_w", q_rank);
+  int dims = 0;
+  const float* csp = nullptr;
+  void* cp = nullptr;
+  if (cache.has_value()) {
+    TORCH_CHECK(act_kind(*cache, "cache") == f && cache->is_contiguous() && cache->dim() == 4 && cache->size(1) == 1 &&
+                cache->size(3) == kv_rank + rot_dim && kv_rank > 0, "latent_prep: cache must be [NB, 1, bs, kv_rank + rot_dim]");
+    TORCH_CHECK(dkv_w.has_value(), "latent_prep: the cached latent needs its norm weight");
+    cp = cache->data_ptr();
+    if (cos_sin.has_value()) {
+      check_f32(*cos_sin, "cos_sin");
+      TORCH_CHECK(cos_sin->dim() == 2 && cos_sin->size(1) <= rot_dim && cos_sin->size(1) % 2 == 0,
+                  "latent_prep: cos_sin must be [max_pos, dims], dims even and at most rot_dim");
+      dims = (int)cos_sin->size(1);
+      csp = cos_sin->data_ptr<float>();
+    }
+  }
+  check_rc(dgi_latent_prep(proj.data_ptr(), (int)proj.stride(0), f, T, (int)q_rank, (int)kv_rank, (int)rot_dim,
+                           dq_w.data_ptr<float>(), cache.has_value() ? f32p(dkv_w, "dkv_w", kv_rank) : nullptr, (float)eps,
+                           i32p(positions, "positions", T), i32p(slots, "slots", T), csp, dims, interleaved ? 1 : 0,
+                           cq.data_ptr(), cp, cur_stream()), "latent_prep");
+}
+
+// [H, T, n] views with unit inner stride: (head stride, row stride)
+void check_htn(const at::Tensor& t, const char* name, int64_t H, int64_t T, int64_t n) {
+  TORCH_CHECK(t.dim() == 3 && t.size(0) == H && t.size(1) == T && t.size(2) == n && (n == 1 || t.stride(2) == 1), name,
+              " must be [H, T, n] with unit inner stride");
+}
+
+void latent_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& q_lat, const at::Tensor& cache,
+                      const at::Tensor& block_tables, const c10::optional<at::Tensor>& cu_seqlens, const at::Tensor& positions,
+                      int64_t H, int64_t dim, int64_t rot_dim, int64_t kv_rank, double scale, int64_t window,
+                      const c10::optional<at::Tensor>& cos_sin, bool interleaved) {
+  const int f = act_kind(q, "q");
+  check_rows(q, "q");
+  const int T = (int)q.size(0);
+  TORCH_CHECK(q.size(1) == H * (dim + rot_dim), "latent_attn_rows: q must be [T, H * (dim + rot_dim)]");
+  TORCH_CHECK(act_kind(q_lat, "q_lat") == f && act_kind(out, "out") == f && act_kind(cache, "cache") == f);
+  check_htn(q_lat, "q_lat", H, T, kv_rank);
+  check_htn(out, "out", H, T, kv_rank);
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 4 && cache.size(1) == 1 && cache.size(3) == kv_rank + rot_dim,
+              "latent_attn_rows: cache must be [NB, 1, bs, kv_rank + rot_dim]");
+  check_i32(block_tables, "block_tables");
+  TORCH_CHECK(block_tables.dim() == 2);
+  const int* cu = nullptr;
+  int n_seqs = (int)block_tables.size(0);
+  if (cu_seqlens.has_value()) {
+    check_i32(*cu_seqlens, "cu_seqlens");
+    n_seqs = (int)cu_seqlens->numel() - 1;
+    TORCH_CHECK(n_seqs >= 1 && n_seqs <= block_tables.size(0), "latent_attn_rows: cu_seqlens does not fit the block tables");
+    cu = cu_seqlens->data_ptr<int>();
+  } else {
+    TORCH_CHECK(block_tables.size(0) >= T, "latent_attn_rows: one block-table row per query row");
+  }
+  int dims = 0;
+  const float* csp = nullptr;
+  if (cos_sin.has_value()) {
+    check_f32(*cos_sin, "cos_sin");
+    TORCH_CHECK(cos_sin->dim() == 2 && cos_sin->size(1) <= rot_dim && cos_sin->size(1) % 2 == 0);
+    dims = (int)cos_sin->size(1);
+    csp = cos_sin->data_ptr<float>();
+  }
+  check_rc(dgi_latent_attn_rows(q.data_ptr(), (int)q.stride(0), q_lat.data_ptr(), (long long)q_lat.stride(0),
+                                (long long)q_lat.stride(1), cache.data_ptr(), block_tables.data_ptr<int>(),
+                                (int)block_tables.stride(0), cu, n_seqs, i32p(positions, "positions", T), T, (int)H, (int)dim,
+                                (int)rot_dim, (int)kv_rank, (int)cache.size(2), (float)scale, (int)window, csp, dims,
+                                interleaved ? 1 : 0, out.data_ptr(), (long long)out.stride(0), (long long)out.stride(1), f,
+                                cur_stream()), "latent_attn_rows");
+}
+
+void gate_heads(at::Tensor out, const at::Tensor& ov, const c10::optional<at::Tensor>& gate, bool per_head) {
+  const int f = act_kind(ov, "ov");
+  TORCH_CHECK(ov.dim() == 3 && (ov.size(2) == 1 || ov.stride(2) == 1), "gate_heads: ov must be [H, T, dv] with unit inner stride");
+  const int H = (int)ov.size(0), T = (int)ov.size(1), dv = (int)ov.size(2);
+  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == (int64_t)H * dv);
+  const void* gp = nullptr;
+  int gs = 0;
+  if (gate.has_value()) {
+    check_rows(*gate, "gate");
+    TORCH_CHECK(act_kind(*gate, "gate") == f && gate->size(0) == T && gate->size(1) == (per_head ? H : H * dv),
+                "gate_heads: gate must be [T, H] (per head) or [T, H * dv]");
+    gp = gate->data_ptr(); gs = (int)gate->stride(0);
+  }
+  check_rc(dgi_gate_heads(out.data_ptr(), ov.data_ptr(), (long long)ov.stride(0), (long long)ov.stride(1), gp, gs,
+                          per_head ? 1 : 0, T, H, dv, f, cur_stream()), "gate_heads");
+}
+
+void gelu_tanh(at::Tensor out, const at::Tensor& x, const c10::optional<at::Tensor>& table,
+               const c10::optional<at::Tensor>& ids, int64_t col0) {
+  const int f = act_kind(x, "x");
+  check_rows(x, "x");
+  TORCH_CHECK(act_kind(out, "out") == f && out.is_contiguous() && out.sizes() == x.sizes());
+  const int T = (int)x.size(0), n = (int)x.size(1);
+  const void* tp = nullptr;
+  const int* ip = nullptr;
+  int ts = 0, vocab = 0;
+  if (table.has_value()) {
+    check_rows(*table, "table");
+    TORCH_CHECK(act_kind(*table, "table") == f && ids.has_value() && col0 >= 0 && col0 + n <= table->size(1),
+                "gelu_tanh: table must hold columns [col0, col0 + n) and come with ids");
+    tp = table->data_ptr(); ts = (int)table->stride(0); vocab = (int)table->size(0);
+    ip = i32p(*ids, "ids", T);
+  }
+  check_rc(dgi_gelu_tanh(out.data_ptr(), x.data_ptr(), (int)x.stride(0), T, n, tp, ts, vocab, ip, (int)col0, f, cur_stream()),
+           "gelu_tanh");
 }
 
 }  // namespace
@@ -511,11 +683,21 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "Tensor positions, Tensor seq_row0, Tensor seq_slots, int heads, int dv, int N, int G, Tensor(c!)? ws=None, "
         "Tensor(d!)? wsd=None, int L=0, int nchunks=0) -> ()");
   m.def("gated_group_norm(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int groups, float eps) -> ()");
-  m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor correction) -> ()");
+  m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor? correction, int sigmoid=0) -> ()");
+  m.def("glu_rows(Tensor(a!) out, Tensor gu, int kind, float limit, float alpha, Tensor? row_scale) -> ()");
+  m.def("stream_add_norm(Tensor(a!) x, Tensor? y, Tensor? post_w, Tensor? next_w, float eps, Tensor(b!)? out) -> ()");
+  m.def("latent_prep(Tensor(a!) cq, Tensor proj, int q_rank, int kv_rank, int rot_dim, Tensor dq_w, Tensor? dkv_w, float eps, "
+        "Tensor positions, Tensor slots, Tensor? cos_sin, bool interleaved, Tensor(b!)? cache) -> ()");
+  m.def("latent_attn_rows(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor cache, Tensor block_tables, Tensor? cu_seqlens, "
+        "Tensor positions, int H, int dim, int rot_dim, int kv_rank, float scale, int window, Tensor? cos_sin, "
+        "bool interleaved) -> ()");
+  m.def("gate_heads(Tensor(a!) out, Tensor ov, Tensor? gate, bool per_head) -> ()");
+  m.def("gelu_tanh(Tensor(a!) out, Tensor x, Tensor? table, Tensor? ids, int col0) -> ()");
   m.def("glu_silu(Tensor(a!) out, Tensor gu) -> ()");
-  m.def("moe_expert_gate_up(Tensor(a!) mid, Tensor h, Tensor idx, Tensor gate_up) -> ()");
+  m.def("moe_expert_gate_up(Tensor(a!) mid, Tensor h, Tensor idx, Tensor gate_up, Tensor? pair_scale=None, int act=0, "
+        "float limit=0.0, float alpha=1.702) -> ()");
   m.def("moe_expert_down(Tensor(a!) ys, Tensor mid, Tensor idx, Tensor down) -> ()");
-  m.def("moe_combine(Tensor(a!) out, Tensor ys, Tensor? where, Tensor h, Tensor idx, Tensor wts, Tensor? shared, int E) -> ()");
+  m.def("moe_combine(Tensor(a!) out, Tensor ys, Tensor? where, Tensor h, Tensor idx, Tensor? wts, Tensor? shared, int E) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
@@ -533,6 +715,12 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("ssm_scan", &ssm_scan);
   m.impl("gated_group_norm", &gated_group_norm);
   m.impl("moe_route", &moe_route);
+  m.impl("glu_rows", &glu_rows);
+  m.impl("stream_add_norm", &stream_add_norm);
+  m.impl("latent_prep", &latent_prep);
+  m.impl("latent_attn_rows", &latent_attn_rows);
+  m.impl("gate_heads", &gate_heads);
+  m.impl("gelu_tanh", &gelu_tanh);
   m.impl("glu_silu", &glu_silu);
   m.impl("moe_expert_gate_up", &moe_expert_gate_up);
   m.impl("moe_expert_down", &moe_expert_down);

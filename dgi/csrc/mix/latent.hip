@@ -1,0 +1,301 @@
+// dgi/csrc/mix/latent.hip — row kernels of latent-attention models on an fp32 residual stream.
+//
+//   stream_add_norm   x += y   (or x += y / rms(y) * post_w)   and   out = x / rms(x) * next_w  (or out = x)
+//                     in one pass over the row: the residual add of one sublayer fused with the RMS
+//                     norm that feeds the next GEMM (the fused_add_rmsnorm of models whose stream is fp32)
+//   latent_prep       row = [query latent | key/value latent | key part | ...] from one fused GEMM:
+//                     RMS norm + weight of the query latent -> cq; RMS norm + weight of the key/value
+//                     latent and rotary of the key part -> one cache row [c | r] in the paged pool
+//   gate_heads        [H, T, dv] head outputs -> [T, H * dv] times sigmoid(gate), one gate per head or per element
+//   gelu_tanh         tanh-form GELU, optionally times a slice of a table row gathered by token id
+//
+// rms(v) = sqrt(mean(v^2) + eps).  Everything is computed in fp32; activations are bf16 or fp32.
+// One 256-thread workgroup per row, the row held in registers between the reduction and the store.
+#include "../common.h"
+
+using namespace dgi;
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, const float* f);
+template <> __device__ __forceinline__ void st4<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t* p, const float* f) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
+}
+
+constexpr int NT = 256;          // threads per row
+constexpr int MAXV = 8;          // 4-column chunks per thread: rows up to NT * 4 * MAXV = 8192 columns
+
+// sum over the workgroup (all threads get it); `red` is NT / 64 floats of LDS, reusable after the call
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();                                   // earlier readers of red are done
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / 64; ++i) s += red[i];
+  return s;
+}
+
+// V = 4: 16-byte accesses (W, strides and pointers allow them); V = 1: any shape
+template <typename TY, typename TO, int V>
+__global__ __launch_bounds__(NT) void stream_add_norm_kernel(float* __restrict__ x, int W, const TY* __restrict__ y,
+                                                             int y_stride, const float* __restrict__ post_w,
+                                                             const float* __restrict__ next_w, float eps,
+                                                             TO* __restrict__ out) {
+  __shared__ float red[NT / 64];
+  const int row = blockIdx.x;
+  float* xr = x + (size_t)row * W;
+  const TY* yr = y ? y + (size_t)row * y_stride : nullptr;
+  float xv[MAXV][V], yv[MAXV][V];
+  float ssy = 0.f;
+#pragma unroll
+  for (int k = 0; k < MAXV; ++k) {
+    const int c = (threadIdx.x + k * NT) * V;
+    if (c < W) {
+      if constexpr (V == 4) {
+        ld4<float>(xr + c, xv[k]);
+        if (yr) ld4<TY>(yr + c, yv[k]);
+      } else {
+        xv[k][0] = xr[c];
+        if (yr) yv[k][0] = ldf<TY>(yr + c);
+      }
+      if (yr) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) ssy += yv[k][j] * yv[k][j];
+      }
+    }
+  }
+  if (yr) {
+    float inv_y = 1.f;
+    if (post_w) inv_y = 1.f / sqrtf(block_sum(ssy, red) / (float)W + eps);
+#pragma unroll
+    for (int k = 0; k < MAXV; ++k) {
+      const int c = (threadIdx.x + k * NT) * V;
+      if (c < W) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) xv[k][j] += post_w ? yv[k][j] * inv_y * post_w[c + j] : yv[k][j];
+        if constexpr (V == 4) st4<float>(xr + c, xv[k]);
+        else xr[c] = xv[k][0];
+      }
+    }
+  }
+  if (!out) return;
+  TO* orow = out + (size_t)row * W;
+  float inv_x = 1.f;
+  if (next_w) {
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < MAXV; ++k) {
+      const int c = (threadIdx.x + k * NT) * V;
+      if (c < W) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) ss += xv[k][j] * xv[k][j];
+      }
+    }
+    inv_x = 1.f / sqrtf(block_sum(ss, red) / (float)W + eps);
+  }
+#pragma unroll
+  for (int k = 0; k < MAXV; ++k) {
+    const int c = (threadIdx.x + k * NT) * V;
+    if (c < W) {
+      float o[V];
+#pragma unroll
+      for (int j = 0; j < V; ++j) o[j] = next_w ? xv[k][j] * inv_x * next_w[c + j] : xv[k][j];
+      if constexpr (V == 4) st4<TO>(orow + c, o);
+      else stf<TO>(orow + c, o[0]);
+    }
+  }
+}
+
+// One workgroup per row.  Query latent: columns [0, q_rank); key/value latent [q_rank, q_rank + kv_rank);
+// key part [q_rank + kv_rank, q_rank + kv_rank + rot_dim), of which the first `dims` rotate.
+template <typename T>
+__global__ __launch_bounds__(NT) void latent_prep_kernel(const T* __restrict__ proj, int stride, int q_rank, int kv_rank,
+                                                         int rot_dim, const float* __restrict__ dq_w,
+                                                         const float* __restrict__ dkv_w, float eps,
+                                                         const int* __restrict__ positions, const int* __restrict__ slots,
+                                                         const float* __restrict__ cos_sin, int dims, int interleaved,
+                                                         T* __restrict__ cq, T* __restrict__ cache) {
+  __shared__ float red[NT / 64];
+  const int row = blockIdx.x;
+  const T* p = proj + (size_t)row * stride;
+  {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < q_rank; c += NT) {
+      const float v = ldf<T>(p + c);
+      ss += v * v;
+    }
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)q_rank + eps);
+    T* o = cq + (size_t)row * q_rank;
+    for (int c = threadIdx.x; c < q_rank; c += NT) stf<T>(o + c, ldf<T>(p + c) * inv * dq_w[c]);
+  }
+  if (!cache) return;
+  const int slot = slots[row];
+  if (slot < 0) return;                               // uniform over the workgroup
+  T* dst = cache + (size_t)slot * (kv_rank + rot_dim);
+  const T* lat = p + q_rank;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < kv_rank; c += NT) {
+    const float v = ldf<T>(lat + c);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)kv_rank + eps);
+  for (int c = threadIdx.x; c < kv_rank; c += NT) stf<T>(dst + c, ldf<T>(lat + c) * inv * dkv_w[c]);
+  const T* kp = lat + kv_rank;
+  T* kd = dst + kv_rank;
+  const int half = dims >> 1;
+  const float* cs = cos_sin ? cos_sin + (size_t)positions[row] * dims : nullptr;
+  for (int i = threadIdx.x; i < half; i += NT) {
+    const int i0 = interleaved ? 2 * i : i, i1 = interleaved ? 2 * i + 1 : i + half;
+    const float u = ldf<T>(kp + i0), v = ldf<T>(kp + i1);
+    const float c = cs[i], s = cs[half + i];
+    stf<T>(kd + i0, u * c - v * s);
+    stf<T>(kd + i1, v * c + u * s);
+  }
+  for (int c = dims + threadIdx.x; c < rot_dim; c += NT) kd[c] = kp[c];
+}
+
+// out[t][h * dv + d] = ov[h][t][d] * sigmoid(gate[t][h] or gate[t][h * dv + d]); grid (T, ceil(H * dv / 256))
+template <typename T>
+__global__ __launch_bounds__(NT) void gate_heads_kernel(T* __restrict__ out, const T* __restrict__ ov, long long ov_hs,
+                                                        long long ov_ts, const T* __restrict__ gate, int gate_stride,
+                                                        int per_head, int H, int dv) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * NT + threadIdx.x;
+  if (c >= H * dv) return;
+  const int h = c / dv, d = c - h * dv;
+  float v = ldf<T>(ov + (size_t)h * ov_hs + (size_t)t * ov_ts + d);
+  if (gate) v *= 1.f / (1.f + expf(-ldf<T>(gate + (size_t)t * gate_stride + (per_head ? h : c))));
+  stf<T>(out + (size_t)t * H * dv + c, v);
+}
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// out[t][c] = gelu(x[t][c]) (* table[ids[t]][col0 + c]); grid-stride over T * n
+template <typename T>
+__global__ __launch_bounds__(NT) void gelu_tanh_kernel(T* __restrict__ out, const T* __restrict__ x, int x_stride, int rows,
+                                                       int n, const T* __restrict__ table, int t_stride, int vocab,
+                                                       const int* __restrict__ ids, int col0) {
+  const size_t total = (size_t)rows * n;
+  for (size_t i = (size_t)blockIdx.x * NT + threadIdx.x; i < total; i += (size_t)gridDim.x * NT) {
+    const size_t r = i / n;
+    const int c = (int)(i - r * n);
+    float v = gelu_tanh_f(ldf<T>(x + r * x_stride + c));
+    if (table) {
+      const int id = min(max(ids[r], 0), vocab - 1);    // no read outside the table
+      v *= ldf<T>(table + (size_t)id * t_stride + col0 + c);
+    }
+    stf<T>(out + i, v);
+  }
+}
+
+template <typename T, int V>
+__global__ __launch_bounds__(NT) void gelu_tanh_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int x_stride,
+                                                           int rows, int n) {
+  const size_t total = (size_t)rows * (n / V);
+  for (size_t i = (size_t)blockIdx.x * NT + threadIdx.x; i < total; i += (size_t)gridDim.x * NT) {
+    const size_t r = i / (n / V);
+    const int c = (int)(i - r * (n / V)) * V;
+    float v[V];
+    ld4<T>(x + r * x_stride + c, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v[j] = gelu_tanh_f(v[j]);
+    st4<T>(out + r * n + c, v);
+  }
+}
+
+}  // namespace
+
+extern "C" int dgi_stream_add_norm(float* x, int T, int W, const void* y, int y_stride, int y_f32, const float* post_w,
+                                   const float* next_w, float eps, void* out, int out_f32, hipStream_t s) {
+  if (T == 0 || W == 0) return 0;
+  if (W > NT * 4 * MAXV) return -3;
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)out) & 15) == 0 &&
+                   W >= NT * 4;       // narrow rows: one column per thread and chunk keeps every thread busy
+#define DGI_SAN(TY_, TO_)                                                                                              \
+  do {                                                                                                                 \
+    if (vec) stream_add_norm_kernel<TY_, TO_, 4><<<T, NT, 0, s>>>(x, W, (const TY_*)y, y_stride, post_w, next_w, eps, (TO_*)out); \
+    else if (W <= NT * MAXV) stream_add_norm_kernel<TY_, TO_, 1><<<T, NT, 0, s>>>(x, W, (const TY_*)y, y_stride, post_w, next_w, eps, (TO_*)out); \
+    else return -4;                                                                                                    \
+  } while (0)
+  if (y_f32) { if (out_f32) DGI_SAN(float, float); else DGI_SAN(float, uint16_t); }
+  else { if (out_f32) DGI_SAN(uint16_t, float); else DGI_SAN(uint16_t, uint16_t); }
+#undef DGI_SAN
+  DGI_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int dgi_latent_prep(const void* proj, int stride, int is_f32, int T, int q_rank, int kv_rank, int rot_dim,
+                               const float* dq_w, const float* dkv_w, float eps, const int* positions, const int* slots,
+                               const float* cos_sin, int dims, int interleaved, void* cq, void* cache, hipStream_t s) {
+  if (T == 0) return 0;
+  if (q_rank <= 0) return -2;
+  if (cache && (kv_rank <= 0 || rot_dim < 0 || dims > rot_dim || (dims & 1) || (dims > 0 && !cos_sin) || !dkv_w || !slots))
+    return -3;
+  if (is_f32)
+    latent_prep_kernel<float><<<T, NT, 0, s>>>((const float*)proj, stride, q_rank, kv_rank, rot_dim, dq_w, dkv_w, eps,
+                                               positions, slots, cos_sin, dims, interleaved, (float*)cq, (float*)cache);
+  else
+    latent_prep_kernel<uint16_t><<<T, NT, 0, s>>>((const uint16_t*)proj, stride, q_rank, kv_rank, rot_dim, dq_w, dkv_w, eps,
+                                                  positions, slots, cos_sin, dims, interleaved, (uint16_t*)cq,
+                                                  (uint16_t*)cache);
+  DGI_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int dgi_gate_heads(void* out, const void* ov, long long ov_hs, long long ov_ts, const void* gate,
+                              int gate_stride, int per_head, int T, int H, int dv, int is_f32, hipStream_t s) {
+  if (T == 0 || H * dv == 0) return 0;
+  const dim3 grid(T, (H * dv + NT - 1) / NT);
+  if (grid.y > 65535) return -3;
+  if (is_f32)
+    gate_heads_kernel<float><<<grid, NT, 0, s>>>((float*)out, (const float*)ov, ov_hs, ov_ts, (const float*)gate,
+                                                 gate_stride, per_head, H, dv);
+  else
+    gate_heads_kernel<uint16_t><<<grid, NT, 0, s>>>((uint16_t*)out, (const uint16_t*)ov, ov_hs, ov_ts,
+                                                    (const uint16_t*)gate, gate_stride, per_head, H, dv);
+  DGI_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int dgi_gelu_tanh(void* out, const void* x, int x_stride, int rows, int n, const void* table, int t_stride,
+                             int vocab, const int* ids, int col0, int is_f32, hipStream_t s) {
+  if (rows == 0 || n == 0) return 0;
+  const bool vec = !table && n % 4 == 0 && x_stride % 4 == 0 && (((uintptr_t)out | (uintptr_t)x) & 15) == 0;
+  const size_t total = (size_t)rows * (vec ? n / 4 : n);
+  const int blocks = (int)((total + NT - 1) / NT > 65535 * 4 ? 65535 * 4 : (total + NT - 1) / NT);
+  if (is_f32) {
+    if (vec) gelu_tanh_vec_kernel<float, 4><<<blocks, NT, 0, s>>>((float*)out, (const float*)x, x_stride, rows, n);
+    else gelu_tanh_kernel<float><<<blocks, NT, 0, s>>>((float*)out, (const float*)x, x_stride, rows, n, (const float*)table,
+                                                       t_stride, vocab, ids, col0);
+  } else {
+    if (vec) gelu_tanh_vec_kernel<uint16_t, 4><<<blocks, NT, 0, s>>>((uint16_t*)out, (const uint16_t*)x, x_stride, rows, n);
+    else gelu_tanh_kernel<uint16_t><<<blocks, NT, 0, s>>>((uint16_t*)out, (const uint16_t*)x, x_stride, rows, n,
+                                                          (const uint16_t*)table, t_stride, vocab, ids, col0);
+  }
+  DGI_CHECK_LAUNCH();
+  return 0;
+}

@@ -1,0 +1,270 @@
+// dgi/csrc/mix/latent_attention.hip — softmax attention over cached latents, for decode rows and
+// prompt rows alike, in bf16 or fp32.
+//
+// The cache holds ONE row per token, [c | r]: the normalised key/value latent c (kr dims) and a
+// rotated key part r (rd dims) that all heads share.  With the unrotated query part folded through
+// the key up-projection beforehand (q_lat [H, T, kr]) head h's score of key j is
+//
+//     s = (q_lat[h] . c_j + rot(q_rot[h]) . r_j) * scale
+//
+// and its output the probability-weighted sum of the c_j (the value up-projection follows as a
+// batched GEMM).  So every head reads the same cached row, as key and as value.  A workgroup
+// therefore owns one query row and a group of heads, one wave per head: tiles of KT cached rows
+// are staged in LDS once (16-byte copies, rows padded against bank conflicts) and every wave
+// scores them (lane j: key j of the tile) and accumulates its weighted sum from LDS (lane l: E
+// consecutive latent dims, one 16-byte LDS read per key).  The row's visible keys are
+//
+//     [max(0, p - window + 1), p]   (window > 0: the last `window` positions, itself included)
+//     [0, p]                        (window == 0)
+//
+// read straight from the pages (this step's rows are written before the kernel runs), so the
+// result does not depend on how a prompt was cut into steps or on what else is in the batch.
+// The query's rotated part is rotated here, while it is staged (interleaved pairs or halves).
+// Scores, the online softmax and the accumulation are fp32; exp is the accurate expf.
+#include "../common.h"
+
+using namespace dgi;
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// E elements (16 bytes) as floats
+template <typename T> __device__ __forceinline__ void ld16(const T* p, float* f);
+template <> __device__ __forceinline__ void ld16<uint16_t>(const uint16_t* p, float* f) {
+  unpack8(*reinterpret_cast<const u32x4*>(p), f);
+}
+template <> __device__ __forceinline__ void ld16<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+
+// VEC: 16-byte accesses (kr and kr + rd multiples of E = 16 / sizeof(T), aligned cache); else element-wise.
+// KT keys per tile (<= 64).  Value chunks per lane: VEC: kr <= 64 * E * MAXC; scalar: kr <= 64 * MAXC.
+template <typename T, bool VEC, int KT>
+__global__ __launch_bounds__(1024) void latent_attn_rows_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ q_lat, long long ql_hs, long long ql_ts,
+    const T* __restrict__ cache, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ cu_seqlens, int n_seqs, const int* __restrict__ positions, int H, int dim, int rd, int kr,
+    int bs, float scale, int window, const float* __restrict__ cos_sin, int dims, int interleaved, T* __restrict__ out,
+    long long o_hs, long long o_ts, int DP, int DQ) {
+  constexpr int E = 16 / sizeof(T);
+  constexpr int CE = VEC ? E : 1;                    // elements per value chunk
+  constexpr int MAXC = VEC ? (sizeof(T) == 2 ? 2 : 4) : 8;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int nw = blockDim.x >> 6;
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  T* tile = reinterpret_cast<T*>(smem);                                  // [KT][DP]
+  float* qs = smem + ((size_t)KT * DP * sizeof(T) + 3) / 4;               // [nw][DQ]
+  float* ps = qs + (size_t)nw * DQ;                                       // [nw][KT]
+  const int D = kr + rd;
+  const int row = blockIdx.x;
+  const int head_raw = blockIdx.y * nw + w;
+  const int head = min(head_raw, H - 1);            // a spare wave shadows the last head and stores nothing
+
+  int seq = row;
+  if (cu_seqlens) {
+    int lo = 0, hi = n_seqs - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (cu_seqlens[mid] <= row) lo = mid; else hi = mid - 1;
+    }
+    seq = lo;
+  }
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const int pos = positions[row];
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+
+  // this wave's query: folded part, then the rotated part
+  float* qw = qs + (size_t)w * DQ;
+  {
+    const T* ql = q_lat + (size_t)head * ql_hs + (size_t)row * ql_ts;
+    for (int e = lane; e < kr; e += 64) qw[e] = ldf<T>(ql + e);
+    const T* qr = q + (size_t)row * q_stride + (size_t)head * (dim + rd) + dim;
+    const int half = dims >> 1;
+    const float* cs = cos_sin ? cos_sin + (size_t)pos * dims : nullptr;
+    for (int i = lane; i < half; i += 64) {
+      const int i0 = interleaved ? 2 * i : i, i1 = interleaved ? 2 * i + 1 : i + half;
+      const float u = ldf<T>(qr + i0), v = ldf<T>(qr + i1);
+      const float c = cs[i], s = cs[half + i];
+      qw[kr + i0] = u * c - v * s;
+      qw[kr + i1] = v * c + u * s;
+    }
+    for (int e = dims + lane; e < rd; e += 64) qw[kr + e] = ldf<T>(qr + e);
+  }
+
+  float m_run = -__builtin_inff(), l_run = 0.f;
+  float o[MAXC][CE];
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c)
+#pragma unroll
+    for (int j = 0; j < CE; ++j) o[c][j] = 0.f;
+  const int nchunk = (kr + CE - 1) / CE;            // value chunks of the latent
+
+  for (int k0 = first; k0 <= pos; k0 += KT) {
+    const int n = min(KT, pos - k0 + 1);
+    __syncthreads();                                 // the previous tile is fully read (and qs written)
+    if constexpr (VEC) {
+      const int cpr = D / E;
+      for (int i = threadIdx.x; i < n * cpr; i += blockDim.x) {
+        const int j = i / cpr, c = i - j * cpr;
+        const int key = k0 + j;
+        const long long slot = (long long)bt[key / bs] * bs + (key % bs);
+        *reinterpret_cast<u32x4*>(tile + (size_t)j * DP + c * E) =
+            *reinterpret_cast<const u32x4*>(cache + slot * D + c * E);
+      }
+    } else {
+      for (int i = threadIdx.x; i < n * D; i += blockDim.x) {
+        const int j = i / D, c = i - j * D;
+        const int key = k0 + j;
+        const long long slot = (long long)bt[key / bs] * bs + (key % bs);
+        tile[(size_t)j * DP + c] = cache[slot * D + c];
+      }
+    }
+    __syncthreads();
+    float s = -__builtin_inff();
+    const bool ok = lane < n;
+    if (ok) {
+      const T* kp = tile + (size_t)lane * DP;
+      float acc = 0.f;
+      if constexpr (VEC) {
+        for (int e = 0; e < D; e += E) {
+          float f[E];
+          ld16<T>(kp + e, f);
+#pragma unroll
+          for (int j = 0; j < E; ++j) acc += qw[e + j] * f[j];
+        }
+      } else {
+        for (int e = 0; e < D; ++e) acc += qw[e] * ldf<T>(kp + e);
+      }
+      s = acc * scale;
+    }
+    const float m_new = fmaxf(m_run, wave_max(s));     // lane 0's key k0 is always visible: finite
+    const float p = ok ? expf(s - m_new) : 0.f;
+    const float corr = expf(m_run - m_new);            // first tile: exp(-inf) = 0
+    l_run = l_run * corr + wave_sum(p);
+    m_run = m_new;
+    float* pw = ps + (size_t)w * KT;
+    if (lane < KT) pw[lane] = p;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // this wave's ps writes precede its reads below
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int ci = lane + 64 * c;
+      if (ci < nchunk) {
+        float acc[CE];
+#pragma unroll
+        for (int j = 0; j < CE; ++j) acc[j] = o[c][j] * corr;
+        const T* vp = tile + (size_t)ci * CE;
+        for (int j = 0; j < n; ++j) {
+          const float pj = pw[j];
+          if constexpr (VEC) {
+            float f[E];
+            ld16<T>(vp + (size_t)j * DP, f);
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[e] += pj * f[e];
+          } else {
+            acc[0] += pj * ldf<T>(vp + (size_t)j * DP);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < CE; ++j) o[c][j] = acc[j];
+      }
+    }
+  }
+  if (head_raw >= H) return;
+  const float inv = 1.f / l_run;
+  T* op = out + (size_t)head * o_hs + (size_t)row * o_ts;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int ci = lane + 64 * c;
+    if (ci < nchunk) {
+#pragma unroll
+      for (int j = 0; j < CE; ++j) stf<T>(op + (size_t)ci * CE + j, o[c][j] * inv);
+    }
+  }
+}
+
+template <typename K>
+int allow_lds(K kernel, size_t lds) {
+  return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+}
+
+// LDS a workgroup may take: what the device reports, at most the 160 KB of a CDNA4 compute unit
+size_t lds_max() {
+  static size_t v = 0;
+  if (!v) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || n <= 0)
+      n = 64 * 1024;
+    v = (size_t)n < 160 * 1024 ? (size_t)n : 160 * 1024;
+  }
+  return v;
+}
+
+template <typename T, bool VEC, int KT>
+int launch(const void* q, int q_stride, const void* q_lat, long long ql_hs, long long ql_ts, const void* cache,
+           const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H,
+           int dim, int rd, int kr, int bs, float scale, int window, const float* cos_sin, int dims, int interleaved,
+           void* out, long long o_hs, long long o_ts, int nw, hipStream_t s) {
+  constexpr int E = 16 / sizeof(T);
+  const int D = kr + rd;
+  const int DP = (D + E - 1) / E * E + E;           // padded row: 16-byte aligned, not a multiple of the bank span
+  const int DQ = (D + 3) / 4 * 4;
+  size_t lds;
+  for (;; nw >>= 1) {
+    lds = ((size_t)KT * DP * sizeof(T) + 3) / 4 * 4 + (size_t)nw * DQ * 4 + (size_t)nw * KT * 4;
+    if (lds <= lds_max() || nw == 1) break;
+  }
+  if (lds > lds_max()) return -6;
+  static int allowed = -1;                           // once per kernel instance
+  if (allowed != 0 && lds > 64 * 1024) {
+    allowed = allow_lds(latent_attn_rows_kernel<T, VEC, KT>, lds_max());
+    if (allowed != 0) return allowed;
+  }
+  const dim3 grid(rows, (H + nw - 1) / nw);
+  latent_attn_rows_kernel<T, VEC, KT><<<grid, 64 * nw, lds, s>>>(
+      (const T*)q, q_stride, (const T*)q_lat, ql_hs, ql_ts, (const T*)cache, block_tables, bt_stride, cu_seqlens, n_seqs,
+      positions, H, dim, rd, kr, bs, scale, window, cos_sin, dims, interleaved, (T*)out, o_hs, o_ts, DP, DQ);
+  return 0;
+}
+
+}  // namespace
+
+// q [rows, H * (dim + rd)] (row stride q_stride); q_lat / out [H, rows, kr] with their own head and row strides;
+// cache [NB, 1, bs, kr + rd]; cu_seqlens (n_seqs + 1 row offsets) maps rows to block-table rows, nullptr: row i
+// uses table row i.  num_cus: workgroups are sized so that the grid covers the chip where the step allows.
+extern "C" int dgi_latent_attn_rows(const void* q, int q_stride, const void* q_lat, long long ql_hs, long long ql_ts,
+                                    const void* cache, const int* block_tables, int bt_stride, const int* cu_seqlens,
+                                    int n_seqs, const int* positions, int rows, int H, int dim, int rd, int kr,
+                                    int block_size, float scale, int window, const float* cos_sin, int dims,
+                                    int interleaved, void* out, long long o_hs, long long o_ts, int is_f32,
+                                    hipStream_t s) {
+  if (rows == 0) return 0;
+  if (H <= 0 || kr <= 0 || rd < 0 || dim < 0 || window < 0) return -2;
+  if (dims > rd || (dims & 1) || (dims > 0 && !cos_sin)) return -3;
+  if (H > 65535 * 16) return -4;
+  const int E = is_f32 ? 4 : 8;
+  const bool vec = kr % E == 0 && (kr + rd) % E == 0 && ((uintptr_t)cache & 15) == 0;
+  if (kr > (vec ? 64 * E * (is_f32 ? 4 : 2) : 64 * 8)) return -5;
+  // heads per workgroup: as many as share a staged tile, fewer when the step has too few rows to fill the chip
+  int nw = 16;
+  while (nw > 1 && nw / 2 >= H) nw >>= 1;
+  while (nw > 2 && (long long)rows * ((H + nw - 1) / nw) < 512) nw >>= 1;
+  int rc;
+#define DGI_LA(TT_, VV_, KK_)                                                                                       \
+  rc = launch<TT_, VV_, KK_>(q, q_stride, q_lat, ql_hs, ql_ts, cache, block_tables, bt_stride, cu_seqlens, n_seqs, \
+                             positions, rows, H, dim, rd, kr, block_size, scale, window, cos_sin, dims, interleaved, \
+                             out, o_hs, o_ts, nw, s)
+  if (is_f32) { if (vec) DGI_LA(float, true, 32); else DGI_LA(float, false, 32); }
+  else { if (vec) DGI_LA(uint16_t, true, 64); else DGI_LA(uint16_t, false, 64); }
+#undef DGI_LA
+  if (rc != 0) return rc;
+  DGI_CHECK_LAUNCH();
+  return 0;
+}

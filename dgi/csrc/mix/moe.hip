@@ -1,9 +1,12 @@
 // dgi/csrc/mix/moe.hip — mixture-of-experts feed-forward: routing, per-pair expert evaluation for
 // small steps, and the combine of sorted-segment expert outputs for large ones.
 //
-//   moe_route         one wave per token: s = softmax(logits) over all R routes (fp32), the `top` routes
-//                     with the largest s + correction (ties: lowest index), weights = s of those routes
+//   moe_route         one wave per token: s = softmax(logits) over all R routes (fp32) or sigmoid of each, the
+//                     `top` routes with the largest s + correction (ties: lowest index), weights = s of those
 //   silu_mul          silu(g) * u over fused [gate | up] rows
+//   glu_rows          the expert activation with an optional per-row factor on gate and up first (a route
+//                     weight on the expert's input, applied after the linear projections) and the clamped
+//                     sigmoid-GLU form min(g, lim) sigmoid(alpha min(g, lim)) (clamp(u, +-lim) + 1)
 //   moe_expert_gate_up / moe_expert_down   small steps: grid (expert, output tile), each workgroup walks the
 //                     pairs that chose its expert straight from the stacked weights [E, 2 ff, W] / [E, W, ff]
 //                     (see below); identity routes (e >= E) belong to no workgroup
@@ -54,7 +57,7 @@ constexpr int MAXR = 8;      // routes per lane: R <= 512
 
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts,
                                                        const float* __restrict__ logits, int l_stride,
-                                                       const float* __restrict__ corr, int R, int top) {
+                                                       const float* __restrict__ corr, int R, int top, int sigmoid) {
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* lp = logits + (size_t)t * l_stride;
   float s[MAXR], c[MAXR];
@@ -70,15 +73,16 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, fl
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
     const int r = lane + 64 * i;
-    s[i] = r < R ? expf(s[i] - m) : 0.f;
+    if (sigmoid) s[i] = r < R ? 1.f / (1.f + expf(-s[i])) : 0.f;     // independent scores
+    else s[i] = r < R ? expf(s[i] - m) : 0.f;
     sum += s[i];
   }
-  const float inv = 1.f / wave_sum(sum);
+  const float inv = sigmoid ? 1.f : 1.f / wave_sum(sum);
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
     const int r = lane + 64 * i;
     s[i] *= inv;
-    c[i] = r < R ? s[i] + corr[r] : -__builtin_inff();
+    c[i] = r < R ? s[i] + (corr ? corr[r] : 0.f) : -__builtin_inff();
   }
   for (int k = 0; k < top; ++k) {
     float bv = -__builtin_inff();
@@ -134,6 +138,38 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
   }
 }
 
+// expert activation on fp32 pre-activations: kind 0 silu(g) * u; kind 1 the clamped sigmoid-GLU
+__device__ __forceinline__ float expert_act(float g, float u, int kind, float limit, float alpha) {
+  if (kind == 1) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  }
+  return g / (1.f + expf(-g)) * u;
+}
+
+template <typename T, int V>
+__global__ void glu_rows_kernel(T* __restrict__ out, const T* __restrict__ gu, int gu_stride, int rows, int I, int kind,
+                                float limit, float alpha, const float* __restrict__ row_scale) {
+  const size_t n = (size_t)rows * (I / V);
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = i / (I / V), c = (i - r * (I / V)) * V;
+    const float rs = row_scale ? row_scale[r] : 1.f;
+    float g[V], u[V], o[V];
+    if constexpr (V == 4) {
+      ld4<T>(gu + r * gu_stride + c, g);
+      ld4<T>(gu + r * gu_stride + I + c, u);
+    } else {
+      g[0] = ldf<T>(gu + r * gu_stride + c);
+      u[0] = ldf<T>(gu + r * gu_stride + I + c);
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) o[k] = expert_act(g[k] * rs, u[k] * rs, kind, limit, alpha);
+    if constexpr (V == 4) st4<T>(out + r * I + c, o);
+    else stf<T>(out + r * I + c, o[0]);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Expert-major evaluation for small steps: a workgroup owns (expert e, a tile of outputs) and walks
 // the (token, route) pairs that chose e, PG at a time, so the expert's weight rows stream once per
@@ -154,11 +190,12 @@ __device__ __forceinline__ int collect_pairs(const int* __restrict__ idx, int ba
   return *cnt;
 }
 
-// mid[pair][f] = silu(Wg[e][f] . h_t) * (Wu[e][f] . h_t)     gate_up [E, 2 ff, W]
+// mid[pair][f] = act(s Wg[e][f] . h_t, s Wu[e][f] . h_t), s = pair_scale[pair] (null: 1)     gate_up [E, 2 ff, W]
 template <typename T, int PG>
 __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
     float* __restrict__ mid, const T* __restrict__ h, int h_stride, const int* __restrict__ idx,
-    const T* __restrict__ gate_up, int P, int top, int ff, int W) {
+    const T* __restrict__ gate_up, int P, int top, int ff, int W, const float* __restrict__ pair_scale, int act,
+    float limit, float alpha) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   int* list = reinterpret_cast<int*>(sm);             // [CAP]
   T* hs = reinterpret_cast<T*>(sm + CAP);             // [PG][W] in the activation dtype (no rounding: h has it)
@@ -226,7 +263,11 @@ __global__ __launch_bounds__(256) void moe_expert_gate_up_kernel(
 #pragma unroll
         for (int p = 0; p < PG; ++p) {
           const float sg = wave_sum(ag[p]), su = wave_sum(au[p]);
-          if (lane == 0 && p < np) mid[(size_t)list[g0 + p] * ff + f] = sg / (1.f + expf(-sg)) * su;
+          if (lane == 0 && p < np) {
+            const int pair = list[g0 + p];
+            const float ps = pair_scale ? pair_scale[pair] : 1.f;
+            mid[(size_t)pair * ff + f] = expert_act(sg * ps, su * ps, act, limit, alpha);
+          }
         }
       }
     }
@@ -319,7 +360,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   }
   for (int k = 0; k < top; ++k) {
     const int e = idx[(size_t)t * top + k];
-    const float wt = wts[(size_t)t * top + k];
+    const float wt = wts ? wts[(size_t)t * top + k] : 1.f;
     const T* src = (e >= E || e < 0) ? h + (size_t)t * h_stride + w
                                      : ys + (size_t)(where ? where[(size_t)t * top + k] : t * top + k) * W + w;
     if constexpr (V == 4) ld4<T>(src, v);
@@ -334,10 +375,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
 }  // namespace
 
 extern "C" int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const float* corr, int T, int R,
-                             int top, hipStream_t s) {
+                             int top, int sigmoid, hipStream_t s) {
   if (T == 0) return 0;
   if (R > 64 * MAXR || top > R || top < 1) return -2;
-  moe_route_kernel<<<T, 64, 0, s>>>(idx, wts, logits, l_stride, corr, R, top);
+  moe_route_kernel<<<T, 64, 0, s>>>(idx, wts, logits, l_stride, corr, R, top, sigmoid);
   DGI_CHECK_LAUNCH();
   return 0;
 }
@@ -371,8 +412,24 @@ static int allow_lds(K kernel, size_t lds) {
   return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
 }
 
+extern "C" int dgi_glu_rows(void* out, const void* gu, int gu_stride, int rows, int I, int kind, float limit, float alpha,
+                            const float* row_scale, int is_f32, hipStream_t s) {
+  if (rows == 0 || I == 0) return 0;
+  const bool vec = I % 4 == 0 && gu_stride % 4 == 0 && (((uintptr_t)out | (uintptr_t)gu) & 15) == 0;
+  const size_t n = (size_t)rows * (vec ? I / 4 : I);
+  const int blocks = (int)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);
+#define DGI_GR(TT_, VV_) \
+  glu_rows_kernel<TT_, VV_><<<blocks, 256, 0, s>>>((TT_*)out, (const TT_*)gu, gu_stride, rows, I, kind, limit, alpha, row_scale)
+  if (is_f32) { if (vec) DGI_GR(float, 4); else DGI_GR(float, 1); }
+  else { if (vec) DGI_GR(uint16_t, 4); else DGI_GR(uint16_t, 1); }
+#undef DGI_GR
+  DGI_CHECK_LAUNCH();
+  return 0;
+}
+
 extern "C" int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up,
-                                      int T, int E, int top, int ff, int W, int is_f32, hipStream_t s) {
+                                      int T, int E, int top, int ff, int W, const float* pair_scale, int act, float limit,
+                                      float alpha, int is_f32, hipStream_t s) {
   if (T == 0 || E == 0) return 0;
   const size_t es = is_f32 ? 4 : 2;
   const int pg = pick_pg((size_t)W * es);
@@ -385,7 +442,7 @@ extern "C" int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, c
     static const int ok = allow_lds(moe_expert_gate_up_kernel<TT_, PG_>, 96 * 1024);                            \
     if (ok != 0) return ok;                                                                                     \
     moe_expert_gate_up_kernel<TT_, PG_><<<grid, 256, lds, s>>>(mid, (const TT_*)h, h_stride, idx, (const TT_*)gate_up, \
-                                                              T * top, top, ff, W);                             \
+                                                              T * top, top, ff, W, pair_scale, act, limit, alpha); \
   } while (0)
   if (is_f32) { if (pg == 8) DGI_GU(float, 8); else if (pg == 4) DGI_GU(float, 4); else if (pg == 2) DGI_GU(float, 2); else DGI_GU(float, 1); }
   else { if (pg == 8) DGI_GU(uint16_t, 8); else if (pg == 4) DGI_GU(uint16_t, 4); else if (pg == 2) DGI_GU(uint16_t, 2); else DGI_GU(uint16_t, 1); }

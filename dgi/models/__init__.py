@@ -1,4 +1,5 @@
-from dgi.models.config import BebovikConfig, ModelConfig, PRESETS, TifepelConfig, get_config  # noqa: F401
+from dgi.models.config import (BebovikConfig, DepelixConfig, ModelConfig, PRESETS, TifepelConfig,  # noqa: F401
+                               get_config)
 
 
 def model_class(cfg):
@@ -9,6 +10,9 @@ def model_class(cfg):
     if isinstance(cfg, TifepelConfig):
         from dgi.models.tifepel import TifepelModel
         return TifepelModel
+    if isinstance(cfg, DepelixConfig):
+        from dgi.models.depelix import DepelixModel
+        return DepelixModel
     from dgi.models.llama import LlamaModel
     return LlamaModel
 

@@ -124,11 +124,13 @@ class ModelConfig:
 @dataclasses.dataclass
 class RotarySpec:
     """Rotary position parameters of one attention mixer: the first ``dims`` dimensions of a
-    head rotate in interleaved pairs (2i, 2i+1) at frequency base^(-2i/dims); ``scaling``
-    (factor, low, high, original) rescales the frequencies by wavelength, or None."""
+    head rotate in pairs at frequency base^(-2i/dims) — ``layout`` "interleaved" pairs (2i, 2i+1),
+    "half" pairs (i, i + dims/2); ``scaling`` (factor, low, high, original) rescales the
+    frequencies by wavelength, or None."""
     base: float
     dims: int
     scaling: Optional[dict] = None
+    layout: str = "interleaved"
 
 
 @dataclasses.dataclass
@@ -220,13 +222,21 @@ class MoeSpec:
     """Mixture-of-experts feed-forward: ``experts`` gated-SiLU experts of width ``ff`` plus
     ``identity`` experts that return their input; a token takes the ``top`` experts with the
     largest softmax score + selection bias and weighs them by the plain scores (not
-    renormalised).  ``shared_ff`` > 0: a shared expert of that width runs for every token."""
+    renormalised).  ``shared_ff`` > 0: a shared expert of that width runs for every token.
+    ``score`` "sigmoid": independent sigmoid scores instead of the softmax.  ``act`` "clamped":
+    experts are clamped sigmoid-GLUs (``GluSpec`` with ``limit``) instead of gated SiLU.
+    ``weigh`` "input": the route weight multiplies the expert's input, not its output."""
     experts: int
     identity: int
     top: int
     ff: int
     shared_ff: int = 0
     kind: str = "moe"
+    score: str = "softmax"
+    act: str = "silu"
+    limit: float = 0.0
+    weigh: str = "output"
+    selection_bias: bool = True     # a learned per-route bias is added to the scores for the choice only
 
     @property
     def routes(self) -> int:
@@ -234,10 +244,67 @@ class MoeSpec:
 
 
 @dataclasses.dataclass
+class LatentAttentionSpec:
+    """One latent-attention mixer: queries go through a normalised latent of ``q_rank`` dims, keys
+    and values of all ``heads`` come from one normalised latent of ``kv_rank`` dims per token plus
+    one rotated key part of ``rot_dim`` dims shared by the heads (the cache holds these two, not
+    per-head keys and values).  A head's query/key has ``dim`` unrotated and ``rot_dim`` rotated
+    dims, its value ``vdim``.  ``mask_kind`` "window": position i sees j with 0 <= i - j <
+    ``mask_size``; "causal": every j <= i.  ``gate`` "head": one sigmoid gate per head, "elem": one
+    per output element, "none".  ``kv_from`` = j: the layer has no latent projection of its own and
+    reads layer j's cached latent and rotated key part."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    scale: float
+    rot: Optional[RotarySpec] = None
+    mask_kind: str = "causal"
+    mask_size: int = 0
+    gate: str = "none"
+    kv_from: Optional[int] = None
+
+    @property
+    def qk_dim(self) -> int:
+        return self.dim + self.rot_dim
+
+    @property
+    def q_size(self) -> int:
+        return self.heads * self.qk_dim
+
+    @property
+    def o_size(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def cache_dim(self) -> int:
+        """Cached elements per token: latent | rotated key part."""
+        return self.kv_rank + self.rot_dim
+
+    @property
+    def gate_rows(self) -> int:
+        return {"head": self.heads, "elem": self.o_size, "none": 0}[self.gate]
+
+    @property
+    def window(self) -> int:
+        return self.mask_size if self.mask_kind == "window" else 0
+
+
+@dataclasses.dataclass
+class DenseSpec:
+    """Plain two-matrix feed-forward W_down act(W_up h); ``act`` "gelu_tanh"."""
+    ff: int
+    act: str = "gelu_tanh"
+    kind: str = "dense"
+
+
+@dataclasses.dataclass
 class LayerSpec:
     type: str
-    mixer: object                     # AttentionSpec | Mamba2Spec
-    mlp: Optional[object] = None      # GluSpec | MoeSpec
+    mixer: object                     # AttentionSpec | Mamba2Spec | LatentAttentionSpec
+    mlp: Optional[object] = None      # GluSpec | MoeSpec | DenseSpec
 
 
 @dataclasses.dataclass
@@ -490,7 +557,163 @@ def tifepel_uniform(name: str, vocab: int, width: int, pattern: str, heads: int,
     return TifepelConfig(name=name, vocab_size=vocab, hidden_size=width, layers=layers, **kw)
 
 
-NATIVE_CONFIGS = {"bebovik": BebovikConfig.from_dict, "tifepel": TifepelConfig.from_dict}
+@dataclasses.dataclass
+class DepelixConfig:
+    """A Depelix decoder: token + hashed-bigram embedding, pre-norm RMS layers on one fp32
+    stream, latent-attention mixers of two kinds (sliding-window with half-split rotary and a
+    per-head gate, possibly reading another layer's cached latent; causal with interleaved rotary
+    and an element gate), dense GELU or sigmoid-routed mixture-of-experts feed-forwards (or
+    none), and after every layer a small per-layer token input (``side_dim`` columns of one
+    shared token table per layer, gated by the stream).  Every layer carries its own sizes."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: list
+    side_dim: int = 0
+    bigram_buckets: int = 0
+    bigram_mul_prev: int = 0
+    bigram_mul_cur: int = 0
+    norm_eps: float = 1e-6
+    max_position: int = 8192
+    bos_token_id: int = -1
+    eos_token_id: int = -1
+    arch: str = "depelix"
+    tie_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def num_heads(self) -> int:
+        return max(l.mixer.heads for l in self.layers)
+
+    @property
+    def num_kv_heads(self) -> int:
+        return 1
+
+    @property
+    def head_dim(self) -> int:
+        return max(l.mixer.cache_dim for l in self.layers)
+
+    @property
+    def rms_eps(self) -> float:
+        return self.norm_eps
+
+    @property
+    def kv_owners(self) -> list:
+        """Layers that write cache pages (those with a latent projection of their own)."""
+        return [i for i, l in enumerate(self.layers) if l.mixer.kv_from is None]
+
+    def kv_layer_shapes(self, start: int = 0, end: Optional[int] = None) -> list:
+        """(1, latent + rotated key part, 0) per layer that owns pages: one shared row per token
+        serves as key and value of every head; layers that read another layer's latent own none."""
+        return [(1, self.layers[i].mixer.cache_dim, 0) for i in self.kv_owners]
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2, layers: Optional[int] = None) -> int:
+        return sum(g * (dk + dv) for g, dk, dv in self.kv_layer_shapes()) * dtype_bytes
+
+    def param_count(self) -> int:
+        W = self.hidden_size
+        n = 2 * self.vocab_size * W + (self.bigram_buckets + 1) * W * bool(self.bigram_buckets)
+        n += self.vocab_size * self.side_dim * len(self.layers)
+        for l in self.layers:
+            m = l.mixer
+            n += W * (m.q_rank + m.gate_rows) + m.q_rank * m.q_size + m.heads * (m.dim + m.vdim) * m.kv_rank + m.o_size * W
+            if m.kv_from is None:
+                n += W * m.cache_dim
+            f = l.mlp
+            if f is not None:
+                n += 2 * W * f.ff if f.kind == "dense" else f.experts * (3 * W * f.ff + W)
+            n += 2 * W * self.side_dim
+        return n
+
+    def to_dict(self) -> dict:
+        return dataclasses.asdict(self)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "depelix") -> "DepelixConfig":
+        kinds = {"latent_attention": ("half", "head"), "latent_attention_2": ("interleaved", "elem")}
+        layers = []
+        for i, e in enumerate(d["layers"]):
+            if e["type"] not in kinds:
+                raise ValueError(f"Depelix: unknown mixer type {e['type']!r}")
+            layout, gate = kinds[e["type"]]
+            m = e["mixer"]
+            rot = m.get("rot") or {}
+            mask = m.get("mask") or {}
+            rot_dim = int(m["rot_dim"])
+            spec = LatentAttentionSpec(
+                heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim, vdim=int(m["vdim"]),
+                kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), scale=float(m["scale"]),
+                rot=RotarySpec(float(rot.get("base", 10000.0)), int(rot.get("dims", rot_dim)), None, layout),
+                mask_kind="window" if mask.get("size") else "causal", mask_size=int(mask.get("size") or 0),
+                gate=gate, kv_from=None if m.get("kv_from") is None else int(m["kv_from"]))
+            if spec.rot.dims > rot_dim or spec.rot.dims % 2:
+                raise ValueError("Depelix: rot.dims must be even and at most rot_dim")
+            if spec.kv_from is not None:
+                j = spec.kv_from
+                if not 0 <= j < i or layers[j].mixer.kv_from is not None:
+                    raise ValueError(f"Depelix: layer {i} reads the latent of layer {j}, which must be an earlier layer "
+                                     "with a latent projection of its own")
+                o = layers[j].mixer
+                if (o.kv_rank, o.rot_dim) != (spec.kv_rank, spec.rot_dim):
+                    raise ValueError(f"Depelix: layers {i} and {j} share a latent but differ in its sizes")
+            f = e.get("mlp")
+            mlp = None
+            if f is not None:
+                kind = f.get("kind", "dense")
+                if kind == "dense":
+                    mlp = DenseSpec(int(f["ff"]))
+                elif kind == "moe":
+                    r = f["router"]
+                    mlp = MoeSpec(experts=int(r["experts"]), identity=0, top=int(r["top"]), ff=int(f["expert"]["ff"]),
+                                  score="sigmoid", act="clamped", limit=float(f["expert"]["limit"]), weigh="input",
+                                  selection_bias=False)
+                    if not 1 <= mlp.top <= mlp.experts:
+                        raise ValueError("Depelix: router.top must be between 1 and router.experts")
+                else:
+                    raise ValueError(f"Depelix: unknown feed-forward kind {kind!r}")
+            layers.append(LayerSpec(e["type"], spec, mlp))
+        bg = (d.get("embedding") or {}).get("bigram") or {}
+        return DepelixConfig(
+            name=name, vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), layers=layers,
+            side_dim=int((d.get("token_side") or {}).get("dim") or 0),
+            bigram_buckets=int(bg.get("buckets") or 0), bigram_mul_prev=int(bg.get("mul_prev") or 0),
+            bigram_mul_cur=int(bg.get("mul_cur") or 0), norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)))
+
+
+def depelix_uniform(name: str, vocab: int, width: int, pattern: str, heads: int, dim: int, rot_dim: int, vdim: int,
+                    kv_rank: int, q_rank: int, window: int, ff: int, experts: int = 0, top: int = 1, expert_ff: int = 0,
+                    limit: float = 7.0, side_dim: int = 0, base: float = 10000.0, **kw) -> DepelixConfig:
+    """A Depelix configuration from a layer pattern: 'w' windowed latent attention, 's' the same
+    reading the latent of the nearest earlier 'w' layer, 'c' causal latent attention; upper case:
+    the layer's feed-forward is a mixture of experts (else dense, ``ff`` 0: none).  All layers of
+    a kind share one geometry (presets, benchmarks)."""
+    layers = []
+    owner = None
+    for i, ch in enumerate(pattern):
+        k = ch.lower()
+        first = k in ("w", "s")
+        if k == "w":
+            owner = i
+        if k == "s" and owner is None:
+            raise ValueError("depelix_uniform: 's' needs an earlier 'w' layer")
+        mixer = LatentAttentionSpec(heads, dim, rot_dim, vdim, kv_rank, q_rank, (dim + rot_dim) ** -0.5,
+                                    RotarySpec(base, rot_dim, None, "half" if first else "interleaved"),
+                                    "window" if first and window else "causal", window if first else 0,
+                                    "head" if first else "elem", owner if k == "s" else None)
+        if ch.isupper() and experts:
+            mlp = MoeSpec(experts, 0, top, expert_ff, score="sigmoid", act="clamped", limit=limit, weigh="input",
+                          selection_bias=False)
+        else:
+            mlp = DenseSpec(ff) if ff else None
+        layers.append(LayerSpec("latent_attention" if first else "latent_attention_2", mixer, mlp))
+    return DepelixConfig(name=name, vocab_size=vocab, hidden_size=width, layers=layers, side_dim=side_dim, **kw)
+
+
+NATIVE_CONFIGS = {"bebovik": BebovikConfig.from_dict, "tifepel": TifepelConfig.from_dict,
+                  "depelix": DepelixConfig.from_dict}
 
 
 PRESETS: dict[str, ModelConfig] = {
@@ -541,6 +764,11 @@ PRESETS: dict[str, ModelConfig] = {
                                     bias_rows=12, bias_max=40.0, norm_groups=2, streams=2, canon_taps=3,
                                     bigram_buckets=251, bigram_mul_prev=31, bigram_mul_cur=7, loop_start=0,
                                     loop_stop=2, loop_times=2, max_position=2048, bos_token_id=1, eos_token_id=2),
+    # Depelix test / smoke sizes (random weights): windowed + shared-latent + causal latent attention,
+    # dense and expert feed-forwards, per-layer token input
+    "depelix-tiny": depelix_uniform("depelix-tiny", 512, 128, "wScW", 4, 16, 16, 24, 48, 64, 40, 256, experts=6, top=2,
+                                    expert_ff=64, limit=2.0, side_dim=16, bigram_buckets=251, bigram_mul_prev=31,
+                                    bigram_mul_cur=7, max_position=2048, bos_token_id=1, eos_token_id=2),
     "opt-125m": ModelConfig(name="opt-125m", arch="opt", vocab_size=50272, hidden_size=768,
                             intermediate_size=3072, num_layers=12, num_heads=12, num_kv_heads=12, head_dim=64,
                             max_position=2048, tie_embeddings=True, bos_token_id=2, eos_token_id=2),
@@ -570,7 +798,7 @@ def get_config(name_or_path: str) -> ModelConfig:
     if "@L" in name_or_path:
         base, n = name_or_path.rsplit("@L", 1)
         bc = get_config(base)
-        if isinstance(bc, (BebovikConfig, TifepelConfig)):
+        if isinstance(bc, (BebovikConfig, TifepelConfig, DepelixConfig)):
             return dataclasses.replace(bc, name=name_or_path, layers=bc.layers[: int(n)])
         return dataclasses.replace(bc, name=name_or_path, num_layers=int(n))
     key = ALIASES.get(name_or_path, name_or_path)

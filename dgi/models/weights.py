@@ -299,3 +299,63 @@ def load_tifepel_checkpoint(model, path: str) -> dict:
     out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
     rd.close()
     return out
+
+
+def load_depelix_checkpoint(model, path: str) -> dict:
+    """Fill a ``DepelixModel`` from the design's safetensors layout: ``embed`` / ``bigram`` / ``side.embed`` /
+    ``head`` / ``final.norm`` and per layer i ``l<i>.norm{1,2}``, the mixer under ``l<i>.mix.`` (dq, dq.norm, uq,
+    dkv, dkv.norm — absent in a layer that reads another layer's latent — uk, uv, g, o), the feed-forward
+    under ``l<i>.mlp.`` (dense: up, down; experts: router, e<j>.{gate,up,down}) and the token input
+    ``l<i>.side.{gate,proj,norm}``.  dq | dkv | g land in one fused weight, every expert's gate | up in one
+    stacked tensor, uk / uv as [heads, rows per head, kv_rank]; norm weights and the router stay fp32."""
+    rd = CheckpointReader(path)
+    n = 0
+
+    def put(dst, name):
+        nonlocal n
+        src = rd.read(name)
+        if tuple(src.shape) != tuple(dst.shape) and src.numel() != dst.numel():
+            raise ValueError(f"{name}: checkpoint shape {tuple(src.shape)} does not fit {tuple(dst.shape)}")
+        _put(dst, src.reshape(dst.shape))
+        n += 1
+
+    for i, L in enumerate(model.layers):
+        p = f"l{i}."
+        m, f = L.spec.mixer, L.spec.mlp
+        put(L.norm1, p + "norm1")
+        r = 0
+        parts = [("dq", m.q_rank)] + ([("dkv", m.cache_dim)] if m.kv_from is None else []) + \
+                ([("g", m.gate_rows)] if m.gate_rows else [])
+        for key, rows in parts:
+            put(L.in_proj[r:r + rows], p + "mix." + key)
+            r += rows
+        put(L.dq_norm, p + "mix.dq.norm")
+        if m.kv_from is None:
+            put(L.dkv_norm, p + "mix.dkv.norm")
+        for dst, key in ((L.uq, "uq"), (L.uk, "uk"), (L.uv, "uv"), (L.o, "o")):
+            put(dst, p + "mix." + key)
+        if f is not None:
+            put(L.norm2, p + "norm2")
+            if f.kind == "dense":
+                put(L.up, p + "mlp.up")
+                put(L.down, p + "mlp.down")
+            else:
+                put(L.router, p + "mlp.router")
+                for e in range(f.experts):
+                    put(L.gate_up[e, : f.ff], f"{p}mlp.e{e}.gate")
+                    put(L.gate_up[e, f.ff:], f"{p}mlp.e{e}.up")
+                    put(L.down[e], f"{p}mlp.e{e}.down")
+        if L.side_gate is not None:
+            put(L.side_gate, p + "side.gate")
+            put(L.side_proj, p + "side.proj")
+            put(L.side_norm, p + "side.norm")
+    put(model.embed, "embed")
+    if model.bigram is not None:
+        put(model.bigram, "bigram")
+    if model.side_embed is not None:
+        put(model.side_embed, "side.embed")
+    put(model.head, "head")
+    put(model.final_norm, "final.norm")
+    out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
+    rd.close()
+    return out
