@@ -77,7 +77,7 @@ def glu_rows(gu: torch.Tensor, act: str = "silu", limit: float = 0.0, alpha: flo
 def moe_route_ref(logits, correction, top, score="softmax"):
     s = torch.softmax(logits.float(), -1) if score == "softmax" else torch.sigmoid(logits.float())
     pick = s if correction is None else s + correction
-    idx = torch.topk(pick, top, dim=-1).indices
+    idx = torch.sort(pick, dim=-1, descending=True, stable=True).indices[:, :top]      # ties: the lowest index first
     return idx.to(torch.int32), torch.gather(s, 1, idx)
 
 
