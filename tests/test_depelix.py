@@ -599,3 +599,15 @@ def test_kernels_match_the_reference_ops_on_a_prompt_batch(dtype, variant):
         close(y, x, 3e-4)
     else:
         assert (y - x).abs().amax(1).median().item() < 0.1
+
+
+def test_bench_arch_compare_option_runs():
+    """`bench.py --arch-compare depelix` (tiny size, CPU): one JSON line with a row per model and phase numbers."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--arch-compare", "depelix", "--arch-sizes", "tiny",
+                        "--prompt-len", "40", "--concurrency", "2", "--steps", "2", "--warmup", "1",
+                        "--max-batched-tokens", "128"], capture_output=True, text=True, timeout=600,
+                       env={**os.environ, "CUDA_VISIBLE_DEVICES": "", "HIP_VISIBLE_DEVICES": ""})
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert [x["model"] for x in out["rows"]] == ["depelix", "llama"]
+    assert all(x["prefill_tok_s"] > 0 and x["decode_tok_s"] > 0 for x in out["rows"])
