@@ -59,6 +59,8 @@ int dgi_stream_add_norm(float* x, int T, int W, const void* y, int y_stride, int
 int dgi_latent_prep(const void* proj, int stride, int is_f32, int T, int q_rank, int kv_rank, int rot_dim,
                     const float* dq_w, const float* dkv_w, float eps, const int* positions, const int* slots,
                     const float* cos_sin, int dims, int interleaved, void* cq, void* cache, hipStream_t s);
+int dgi_rotate_heads(void* x, int stride, int is_f32, int T, const int* positions, const float* cos_sin, int dims,
+                     int interleaved, int H, int hs, int off, hipStream_t s);
 int dgi_gate_heads(void* out, const void* ov, long long ov_hs, long long ov_ts, const void* gate, int gate_stride,
                    int per_head, int T, int H, int dv, int is_f32, hipStream_t s);
 int dgi_gelu_tanh(void* out, const void* x, int x_stride, int rows, int n, const void* table, int t_stride, int vocab,
@@ -618,6 +620,17 @@ void latent_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& q_l
                                 cur_stream()), "latent_attn_rows");
 }
 
+void rotate_heads(at::Tensor x, const at::Tensor& positions, const at::Tensor& cos_sin, bool interleaved, int64_t H,
+                  int64_t head_size, int64_t offset) {
+  const int f = act_kind(x, "x");
+  check_rows(x, "x");
+  check_f32(cos_sin, "cos_sin");
+  TORCH_CHECK(cos_sin.dim() == 2 && x.size(1) >= H * head_size, "rotate_heads: x rows hold H heads of head_size");
+  check_rc(dgi_rotate_heads(x.data_ptr(), (int)x.stride(0), f, (int)x.size(0), i32p(positions, "positions", x.size(0)),
+                            cos_sin.data_ptr<float>(), (int)cos_sin.size(1), interleaved ? 1 : 0, (int)H, (int)head_size,
+                            (int)offset, cur_stream()), "rotate_heads");
+}
+
 void gate_heads(at::Tensor out, const at::Tensor& ov, const c10::optional<at::Tensor>& gate, bool per_head) {
   const int f = act_kind(ov, "ov");
   TORCH_CHECK(ov.dim() == 3 && (ov.size(2) == 1 || ov.stride(2) == 1), "gate_heads: ov must be [H, T, dv] with unit inner stride");
@@ -691,6 +704,7 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
   m.def("latent_attn_rows(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor cache, Tensor block_tables, Tensor? cu_seqlens, "
         "Tensor positions, int H, int dim, int rot_dim, int kv_rank, float scale, int window, Tensor? cos_sin, "
         "bool interleaved) -> ()");
+  m.def("rotate_heads(Tensor(a!) x, Tensor positions, Tensor cos_sin, bool interleaved, int H, int head_size, int offset) -> ()");
   m.def("gate_heads(Tensor(a!) out, Tensor ov, Tensor? gate, bool per_head) -> ()");
   m.def("gelu_tanh(Tensor(a!) out, Tensor x, Tensor? table, Tensor? ids, int col0) -> ()");
   m.def("glu_silu(Tensor(a!) out, Tensor gu) -> ()");
@@ -719,6 +733,7 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("stream_add_norm", &stream_add_norm);
   m.impl("latent_prep", &latent_prep);
   m.impl("latent_attn_rows", &latent_attn_rows);
+  m.impl("rotate_heads", &rotate_heads);
   m.impl("gate_heads", &gate_heads);
   m.impl("gelu_tanh", &gelu_tanh);
   m.impl("glu_silu", &glu_silu);

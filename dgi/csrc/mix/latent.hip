@@ -6,6 +6,7 @@
 //   latent_prep       row = [query latent | key/value latent | key part | ...] from one fused GEMM:
 //                     RMS norm + weight of the query latent -> cq; RMS norm + weight of the key/value
 //                     latent and rotary of the key part -> one cache row [c | r] in the paged pool
+//   rotate_heads      rotary on `dims` entries at a fixed offset inside every head of a row, in place
 //   gate_heads        [H, T, dv] head outputs -> [T, H * dv] times sigmoid(gate), one gate per head or per element
 //   gelu_tanh         tanh-form GELU, optionally times a slice of a table row gathered by token id
 //
@@ -176,6 +177,25 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(const T* __restrict__ p
   for (int c = dims + threadIdx.x; c < rot_dim; c += NT) kd[c] = kp[c];
 }
 
+// x[t][h * hs + off + (pair)] rotated by the row's position; grid (T), threads over H * dims / 2 pairs
+template <typename T>
+__global__ __launch_bounds__(NT) void rotate_heads_kernel(T* __restrict__ x, int stride, const int* __restrict__ positions,
+                                                          const float* __restrict__ cos_sin, int dims, int interleaved,
+                                                          int H, int hs, int off) {
+  const int t = blockIdx.x, half = dims >> 1;
+  const float* cs = cos_sin + (size_t)positions[t] * dims;
+  T* row = x + (size_t)t * stride;
+  for (int i = threadIdx.x; i < H * half; i += NT) {
+    const int h = i / half, k = i - h * half;
+    T* p = row + (size_t)h * hs + off;
+    const int i0 = interleaved ? 2 * k : k, i1 = interleaved ? 2 * k + 1 : k + half;
+    const float u = ldf<T>(p + i0), v = ldf<T>(p + i1);
+    const float c = cs[k], sn = cs[half + k];
+    stf<T>(p + i0, u * c - v * sn);
+    stf<T>(p + i1, v * c + u * sn);
+  }
+}
+
 // out[t][h * dv + d] = ov[h][t][d] * sigmoid(gate[t][h] or gate[t][h * dv + d]); grid (T, ceil(H * dv / 256))
 template <typename T>
 __global__ __launch_bounds__(NT) void gate_heads_kernel(T* __restrict__ out, const T* __restrict__ ov, long long ov_hs,
@@ -262,6 +282,16 @@ extern "C" int dgi_latent_prep(const void* proj, int stride, int is_f32, int T, 
     latent_prep_kernel<uint16_t><<<T, NT, 0, s>>>((const uint16_t*)proj, stride, q_rank, kv_rank, rot_dim, dq_w, dkv_w, eps,
                                                   positions, slots, cos_sin, dims, interleaved, (uint16_t*)cq,
                                                   (uint16_t*)cache);
+  DGI_CHECK_LAUNCH();
+  return 0;
+}
+
+extern "C" int dgi_rotate_heads(void* x, int stride, int is_f32, int T, const int* positions, const float* cos_sin, int dims,
+                                int interleaved, int H, int hs, int off, hipStream_t s) {
+  if (T == 0 || dims == 0 || H == 0) return 0;
+  if ((dims & 1) || off < 0 || off + dims > hs || (long long)H * hs > stride) return -2;
+  if (is_f32) rotate_heads_kernel<float><<<T, NT, 0, s>>>((float*)x, stride, positions, cos_sin, dims, interleaved, H, hs, off);
+  else rotate_heads_kernel<uint16_t><<<T, NT, 0, s>>>((uint16_t*)x, stride, positions, cos_sin, dims, interleaved, H, hs, off);
   DGI_CHECK_LAUNCH();
   return 0;
 }

@@ -12,7 +12,7 @@ using namespace dgi;
 using namespace dgi::prefill;
 
 // tiles: int32 [n_tiles, 2] = (sequence index, first query row of the 128-row tile);
-// mask: block size in positions (0 = plain causal); gate: [rows, >= nh * hd] or nullptr
+// mask: block size in positions (0 = plain causal, < 0: a sliding window of -mask positions); gate: [rows, >= nh * hd] or nullptr
 extern "C" int dgi_paged_prefill_masked(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                         const int* block_tables, int bt_stride, const int* cu_seqlens_q,
                                         const int* context_lens, const int* tiles, int n_tiles, void* out,
@@ -21,7 +21,7 @@ extern "C" int dgi_paged_prefill_masked(const void* q, int q_stride, const void*
                                         int n_dist, hipStream_t s) {
   if (n_tiles == 0) return 0;
   if (hd != 128 && hd != 64) return -5;
-  if (nkv <= 0 || nh % nkv || mask < 0) return -2;
+  if (nkv <= 0 || nh % nkv) return -2;
   if (dist_bias && (n_dist < 1 || scale == 0.f)) return -6;
   int bs_log2 = 0;
   while ((1 << bs_log2) < block_size) ++bs_log2;

@@ -2,6 +2,7 @@
 // prefill_attention.hip (plain causal / tree mask) and mix/masked_prefill.hip (block mask +
 // output gate).  See prefill_attention.hip for the tiling; MASKED adds two things:
 //   * a block ("chunk") mask: a query at position p sees keys [floor(p / mask) * mask, p]
+//     (mask < 0: a sliding window, keys [max(0, p + mask + 1), p], i.e. the last -mask positions)
 //     (mask > 0; blocks are counted from position 0 of the sequence, so the result does not
 //     depend on where a prompt was cut).  K/V tiles wholly before the first block of the
 //     workgroup's rows are never loaded, tiles before a wave's first block are skipped, and a
@@ -105,7 +106,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
   const int kv_end = min(ctx, pos_base + last_row + 1);
   // block mask: first visible key of a position; the workgroup starts at the 64-key tile
   // holding the first block of its first row
-  auto first_key = [&](int p) { return (MASKED && mask > 0) ? (p / mask) * mask : 0; };
+  // (mask < 0: a sliding window of -mask positions instead, first key max(0, p + mask + 1))
+  auto first_key = [&](int p) {
+    if (!MASKED || mask == 0) return 0;
+    return mask > 0 ? (p / mask) * mask : max(0, p + mask + 1);
+  };
   const int kv_begin = MASKED ? (first_key(pos_base + t0) / KT) * KT : 0;
   const int my_first = first_key(my_pos);
 

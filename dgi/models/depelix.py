@@ -44,16 +44,20 @@ bigram hash from ``dgi.kv.state_pool.StatePool``.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
 
 from dgi import ops
 from dgi.models.config import DepelixConfig
-from dgi.ops import latent, moe, recur
+from dgi.ops import latent, mix, moe, recur
 from dgi.runtime.batch import AttnMeta
 
 GLU_ALPHA = 1.702          # sigmoid slope of the experts' gate activation (fixed by the design)
+# prompt rows of a step from which the MFMA prompt path (keys and values expanded per head) replaces the
+# row-wise kernel, where the geometry allows it (DGI_LATENT_MFMA_ROWS; a huge value switches it off)
+MFMA_PROMPT_ROWS = int(os.environ.get("DGI_LATENT_MFMA_ROWS", "64"))
 
 
 class DepelixLayerWeights:
@@ -248,10 +252,14 @@ class DepelixModel:
                                 meta.positions, meta.slot_mapping, L.cos_sin, inter, cache if own else None)
         q = ops.linear(cq, L.uq)
         T, H, kr = q.shape[0], m.heads, m.kv_rank
+        nd = meta.num_decode
+        g0 = m.q_rank + (m.cache_dim if own else 0)
+        gate = proj[:, g0:g0 + m.gate_rows] if m.gate_rows else None
+        if meta.num_prefill_tokens >= MFMA_PROMPT_ROWS and self._mfma_prompt_ok(m, q):
+            return ops.linear(self._attention_mfma_prompt(L, m, q, gate, cache, meta, inter), L.o)
         # unrotated query part of every head through its key up-projection: [H, T, dim] x [H, dim, kr]
         q_lat = torch.bmm(q.view(T, H, m.qk_dim)[:, :, :m.dim].transpose(0, 1), L.uk)
         o_lat = torch.empty(H, T, kr, device=q.device, dtype=q.dtype)
-        nd = meta.num_decode
         if nd > 0:
             latent.latent_attn_rows(q[:nd], q_lat[:, :nd], cache, meta.dec_block_tables, None, meta.positions[:nd], H,
                                     m.dim, m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter, out=o_lat[:, :nd])
@@ -260,9 +268,50 @@ class DepelixModel:
                                     meta.positions[nd:], H, m.dim, m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter,
                                     out=o_lat[:, nd:])
         ov = torch.bmm(o_lat, L.uv.transpose(1, 2))                       # weighted latent sums -> head values
-        g0 = m.q_rank + (m.cache_dim if own else 0)
-        gate = proj[:, g0:g0 + m.gate_rows] if m.gate_rows else None
         return ops.linear(latent.gate_heads(ov, gate, m.gate == "head"), L.o)
+
+    @staticmethod
+    def _mfma_prompt_ok(m, q: torch.Tensor) -> bool:
+        return (q.is_cuda and q.dtype == torch.bfloat16 and m.qk_dim == m.vdim and m.vdim in (64, 128)
+                and mix.masked_prefill_available() and not torch.cuda.is_current_stream_capturing())
+
+    def _attention_mfma_prompt(self, L, m, q, gate, cache, meta: AttnMeta, inter: bool) -> torch.Tensor:
+        """Gated head outputs [T, H * vdim] of a step with prompt portions, on the MFMA flash kernel: the
+        portions' pages are expanded once into per-head keys [U_k c | r] and values U_v c (two GEMMs over
+        the cached latents: the explicit form costs (dim + rot_dim + vdim) MACs per query, key and head
+        instead of the 2 kv_rank + rot_dim of the folded form), laid out as pages of their own; the step's
+        decode rows still run the folded row-wise kernel on the cached latents."""
+        T, H, kr, dv = q.shape[0], m.heads, m.kv_rank, m.vdim
+        nd = meta.num_decode
+        out = torch.empty(T, H * dv, device=q.device, dtype=q.dtype)
+        per_head = m.gate == "head"
+        if nd > 0:
+            q_lat = torch.bmm(q[:nd].view(nd, H, m.qk_dim)[:, :, :m.dim].transpose(0, 1), L.uk)
+            o_lat = torch.empty(H, nd, kr, device=q.device, dtype=q.dtype)
+            latent.latent_attn_rows(q[:nd], q_lat, cache, meta.dec_block_tables, None, meta.positions[:nd], H, m.dim,
+                                    m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter, out=o_lat)
+            latent.gate_heads(torch.bmm(o_lat, L.uv.transpose(1, 2)), None if gate is None else gate[:nd], per_head,
+                              out=out[:nd])
+        bt = meta.pre_block_tables
+        Bp, mb = bt.shape
+        bs = cache.shape[2]
+        rows = cache.view(cache.shape[0], bs, m.cache_dim).index_select(0, bt.reshape(-1).long())    # [P, bs, kr + rd]
+        npg = Bp * mb
+        lat = rows.view(npg * bs, m.cache_dim)[:, :kr]
+        kt = torch.empty(npg, H, bs, m.qk_dim, device=q.device, dtype=q.dtype)
+        kt[..., :m.dim] = ops.linear(lat, L.uk.view(H * m.dim, kr)).view(npg, bs, H, m.dim).permute(0, 2, 1, 3)
+        kt[..., m.dim:] = rows[:, None, :, kr:]
+        vt = ops.linear(lat, L.uv.view(H * dv, kr)).view(npg, bs, H, dv).permute(0, 2, 1, 3).contiguous()
+        qp = q[nd:]
+        if L.cos_sin is not None:
+            latent.rotate_heads(qp, meta.positions[nd:], L.cos_sin, inter, H, m.qk_dim, m.dim)
+        own_bt = torch.arange(npg, dtype=torch.int32, device=q.device).view(Bp, mb)
+        att = mix.paged_prefill_masked(qp, kt, vt, own_bt, meta.pre_cu_seqlens, meta.pre_context_lens, H, H, m.scale, 0,
+                                       None if per_head or gate is None else gate[nd:], tiles=meta.pre_tiles,
+                                       window=m.window, out=out[nd:] if not per_head else None)
+        if per_head:
+            latent.gate_heads(att.view(T - nd, H, dv).transpose(0, 1), None if gate is None else gate[nd:], True, out=out[nd:])
+        return out
 
     def _ff(self, L, h: torch.Tensor) -> torch.Tensor:
         f = L.spec.mlp

@@ -175,18 +175,37 @@ def gate_heads_ref(ov, gate, per_head):
     return o.reshape(T, H * dv).to(ov.dtype)
 
 
-def gate_heads(ov: torch.Tensor, gate: Optional[torch.Tensor], per_head: bool) -> torch.Tensor:
-    """Head outputs ``ov`` [H, T, dv] -> [T, H * dv] (heads side by side), multiplied by
-    sigmoid(gate): ``gate`` [T, H] with ``per_head`` (one gate per head), else [T, H * dv]; None: no gate."""
+def gate_heads(ov: torch.Tensor, gate: Optional[torch.Tensor], per_head: bool,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Head outputs ``ov`` [H, T, dv] (any head / row strides) -> [T, H * dv] (heads side by side),
+    multiplied by sigmoid(gate): ``gate`` [T, H] with ``per_head`` (one gate per head), else
+    [T, H * dv]; None: no gate.  ``out``: contiguous rows to write."""
+    H, T, dv = ov.shape
     if _native(ov):
-        H, T, dv = ov.shape
-        out = torch.empty(T, H * dv, dtype=ov.dtype, device=ov.device)
+        if out is None:
+            out = torch.empty(T, H * dv, dtype=ov.dtype, device=ov.device)
         _call("gate_heads", out, ov, gate, bool(per_head))
         return out
-    if gate is None:
-        H, T, dv = ov.shape
-        return ov.permute(1, 0, 2).reshape(T, H * dv).contiguous()
-    return gate_heads_ref(ov, gate, per_head)
+    r = ov.permute(1, 0, 2).reshape(T, H * dv).contiguous() if gate is None else gate_heads_ref(ov, gate, per_head)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+def rotate_heads(x: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor, interleaved: bool, H: int,
+                 head_size: int, offset: int) -> torch.Tensor:
+    """Rotary in place on ``cos_sin.shape[1]`` entries starting at ``offset`` inside each of the H heads
+    (``head_size`` apart) of every row of ``x`` [T, >= H * head_size], by the row's position."""
+    if _native(x):
+        _call("rotate_heads", x, positions, cos_sin, bool(interleaved), int(H), int(head_size), int(offset))
+        return x
+    T, dims = x.shape[0], cos_sin.shape[1]
+    if T:
+        v = x[:, :H * head_size].view(T, H, head_size)
+        r = rotate_ref(v[:, :, offset:offset + dims].float(), cos_sin[positions.long()], dims, interleaved)
+        v[:, :, offset:offset + dims] = r.to(x.dtype)
+    return x
 
 
 # ----------------------------------------------------------------------------

@@ -181,7 +181,7 @@ def distance_bias_table(rel: torch.Tensor, far: float) -> torch.Tensor:
 
 
 def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate=None,
-                         dist_bias=None):
+                         dist_bias=None, window=0):
     T = q.shape[0]
     bs, dk, dv = k_cache.shape[2], k_cache.shape[3], v_cache.shape[3]
     out = torch.zeros(T, H * dv, dtype=q.dtype, device=q.device)
@@ -195,7 +195,7 @@ def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, position
             while cu[seq + 1] <= t:
                 seq += 1
         p = pos[t]
-        first = (p // mask) * mask if mask > 0 else 0
+        first = (p // mask) * mask if mask > 0 else (max(0, p - window + 1) if window > 0 else 0)
         keys = torch.arange(first, p + 1, device=q.device)
         blk = block_tables[seq][keys // bs].long()
         k = k_cache[blk, :, keys % bs].float()          # [n, G, dk]
@@ -247,9 +247,10 @@ def masked_prefill_available() -> bool:
 
 
 def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, nh, nkv, scale,
-                         mask: int = 0, gate=None, tiles=None, out=None, dist_bias=None) -> torch.Tensor:
+                         mask: int = 0, gate=None, tiles=None, out=None, dist_bias=None, window: int = 0) -> torch.Tensor:
     """``paged_prefill`` with a block mask — a query at position p sees keys
-    [floor(p / mask) * mask, p] (``mask`` 0: all keys up to p) — and an optional sigmoid output
+    [floor(p / mask) * mask, p] (``mask`` 0: all keys up to p) — or a sliding window (``window`` > 0
+    with ``mask`` 0: keys [max(0, p - window + 1), p]) and an optional sigmoid output
     gate (out *= sigmoid(gate)) and an optional distance bias (``dist_bias`` as in
     ``masked_attn_rows``).  bf16, key size == value size in {64, 128} on the GPU
     (dgi/csrc/mix/masked_prefill.hip); the row-wise reference elsewhere."""
@@ -261,14 +262,16 @@ def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, contex
         if tiles is None:
             tl = ops.prefill_tiles(cu_seqlens_q.tolist(), context_lens=context_lens.tolist(), tile=128)
             tiles = torch.tensor(tl if tl else [[0, 0]], dtype=torch.int32, device=q.device)[: len(tl)]
+        if mask and window:
+            raise ValueError("paged_prefill_masked: a block mask or a window, not both")
         _call("paged_prefill_masked", out, q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, tiles,
-              nh, nkv, float(scale), int(mask), gate, dist_bias)
+              nh, nkv, float(scale), int(mask) if mask else -int(window), gate, dist_bias)      # the kernel takes a window as a negative mask
         return out
     cu = cu_seqlens_q.tolist()
     pos = torch.cat([torch.arange(int(context_lens[b]) - (cu[b + 1] - cu[b]), int(context_lens[b]), dtype=torch.int32)
                      for b in range(len(cu) - 1)]) if len(cu) > 1 else torch.zeros(0, dtype=torch.int32)
     r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens_q, pos.to(q.device), nh, nkv, scale,
-                             mask, gate, dist_bias)
+                             mask, gate, dist_bias, window)
     if out is not None:
         out.copy_(r)
         return out

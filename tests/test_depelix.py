@@ -611,3 +611,68 @@ def test_bench_arch_compare_option_runs():
     out = json.loads(r.stdout.strip().splitlines()[-1])
     assert [x["model"] for x in out["rows"]] == ["depelix", "llama"]
     assert all(x["prefill_tok_s"] > 0 and x["decode_tok_s"] > 0 for x in out["rows"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hd,H,window", [(64, 4, 100), (128, 2, 64), (128, 3, 1), (64, 2, 300)])
+def test_mfma_prompt_kernel_with_a_sliding_window(hd, H, window):
+    """The MFMA prompt kernel with a sliding window against the row-wise reference: two portions on top of cached
+    tokens, windows that end inside 64-key tiles and span several, a dominating key just inside / outside."""
+    from dgi.ops import mix
+    bs, G = 16, H
+    g = torch.Generator().manual_seed(7)
+    lens, ctx = [200, 77], [330, 77]
+    nblk = sum((c + bs - 1) // bs for c in ctx)
+    kc = (torch.randn(nblk + 1, G, bs, hd, generator=g) * 0.5).to(torch.bfloat16)
+    vc = (torch.randn(nblk + 1, G, bs, hd, generator=g) * 0.5).to(torch.bfloat16)
+    q = (torch.randn(sum(lens), H * hd, generator=g) * 0.5).to(torch.bfloat16)
+    perm = (torch.randperm(nblk, generator=g) + 1).tolist()
+    mb = max((c + bs - 1) // bs for c in ctx)
+    bt = torch.zeros(2, mb, dtype=I32)
+    at = 0
+    for b, c in enumerate(ctx):
+        n = (c + bs - 1) // bs
+        bt[b, :n] = torch.tensor(perm[at:at + n], dtype=I32)
+        at += n
+    # row 150 of the first portion sits at position 280: its window starts at 280 - window + 1
+    p = 280
+    for j, scale in ((p - window + 1, 6.0), (p - window, 9.0)):
+        if j >= 0:
+            kc[int(bt[0, j // bs]), 0, j % bs] = (q[150, :hd].float() * scale).to(torch.bfloat16)
+    cu = torch.tensor([0, lens[0], sum(lens)], dtype=I32)
+    cl = torch.tensor(ctx, dtype=I32)
+    want = mix.paged_prefill_masked(q, kc, vc, bt, cu, cl, H, G, 0.2, 0, None, window=window)            # CPU: row-wise reference
+    got = mix.paged_prefill_masked(q.cuda(), kc.cuda(), vc.cuda(), bt.cuda(), cu.cuda(), cl.cuda(), H, G, 0.2, 0, None,
+                                   window=window)
+    close(got.float(), want.float(), 0.03)
+
+
+@pytest.mark.gpu
+def test_mfma_prompt_path_in_the_model(monkeypatch):
+    """Layers whose bf16 heads are 64 / 128 wide (unrotated + rotated = value size) take the MFMA prompt kernel
+    on expanded keys and values: same logits as the row-wise kernel on the cached latents (portions on top of
+    cached tokens, two prompts and a decode row in one step, windows shorter than the prompt, a shared latent)."""
+    from dgi.models import depelix as dm
+    cfg = DepelixConfig(name="t", vocab_size=53, hidden_size=64, layers=[
+        LayerSpec(T1, la(1, 4, 32, 32, 64, 40, 48, window=70), DenseSpec(64)),
+        LayerSpec(T1, la(1, 2, 64, 64, 128, 40, 32, window=33, kv_from=0), None),
+        LayerSpec(T2, la(2, 3, 96, 32, 128, 24, 32), DenseSpec(64)),
+        LayerSpec(T2, la(2, 2, 16, 48, 64, 24, 32, kv_from=2), None),
+    ], side_dim=8, bigram_buckets=29, bigram_mul_prev=5, bigram_mul_cur=3, max_position=512)
+    a, b, c = toks(200, 70), toks(90, 71), toks(40, 72)
+
+    def run():
+        eng = engine(cfg, "cuda", dtype=torch.bfloat16, num_blocks=64, bs=16, max_len=512)
+        out = [eng.feed([("a", a[:150], list(range(150))), ("c", c[:39], [38])]),
+               eng.feed([("a", a[150:], list(range(50))), ("b", b, list(range(90))), ("c", c[39:], [0])], ["a", "b", "c"])]
+        return torch.cat([o for step in out for o in step], 0)
+
+    calls = []
+    real = dm.DepelixModel._attention_mfma_prompt
+    monkeypatch.setattr(dm.DepelixModel, "_attention_mfma_prompt", lambda self, *a, **k: (calls.append(1), real(self, *a, **k))[1])
+    fast = run()
+    assert len(calls) == 8                                   # every layer of both steps
+    monkeypatch.setattr(dm, "MFMA_PROMPT_ROWS", 1 << 30)
+    slow = run()
+    assert len(calls) == 8
+    close(fast, slow, 0.06 * max(1.0, slow.abs().max().item()))
