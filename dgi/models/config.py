@@ -600,6 +600,19 @@ class DepelixConfig:
     def rms_eps(self) -> float:
         return self.norm_eps
 
+    def __post_init__(self):
+        for i, l in enumerate(self.layers):
+            m = l.mixer
+            if m.kv_from is None:
+                continue
+            j = m.kv_from
+            if not 0 <= j < i or self.layers[j].mixer.kv_from is not None:
+                raise ValueError(f"Depelix: layer {i} reads the latent of layer {j}, which must be an earlier layer "
+                                 "with a latent projection of its own")
+            o = self.layers[j].mixer
+            if (o.kv_rank, o.rot_dim) != (m.kv_rank, m.rot_dim):
+                raise ValueError(f"Depelix: layers {i} and {j} share a latent but differ in its sizes")
+
     @property
     def kv_owners(self) -> list:
         """Layers that write cache pages (those with a latent projection of their own)."""
@@ -651,14 +664,6 @@ class DepelixConfig:
                 gate=gate, kv_from=None if m.get("kv_from") is None else int(m["kv_from"]))
             if spec.rot.dims > rot_dim or spec.rot.dims % 2:
                 raise ValueError("Depelix: rot.dims must be even and at most rot_dim")
-            if spec.kv_from is not None:
-                j = spec.kv_from
-                if not 0 <= j < i or layers[j].mixer.kv_from is not None:
-                    raise ValueError(f"Depelix: layer {i} reads the latent of layer {j}, which must be an earlier layer "
-                                     "with a latent projection of its own")
-                o = layers[j].mixer
-                if (o.kv_rank, o.rot_dim) != (spec.kv_rank, spec.rot_dim):
-                    raise ValueError(f"Depelix: layers {i} and {j} share a latent but differ in its sizes")
             f = e.get("mlp")
             mlp = None
             if f is not None:

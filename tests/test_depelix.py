@@ -655,9 +655,9 @@ def test_mfma_prompt_path_in_the_model(monkeypatch):
     from dgi.models import depelix as dm
     cfg = DepelixConfig(name="t", vocab_size=53, hidden_size=64, layers=[
         LayerSpec(T1, la(1, 4, 32, 32, 64, 40, 48, window=70), DenseSpec(64)),
-        LayerSpec(T1, la(1, 2, 64, 64, 128, 40, 32, window=33, kv_from=0), None),
+        LayerSpec(T1, la(1, 2, 96, 32, 128, 40, 32, window=33, kv_from=0), None),
         LayerSpec(T2, la(2, 3, 96, 32, 128, 24, 32), DenseSpec(64)),
-        LayerSpec(T2, la(2, 2, 16, 48, 64, 24, 32, kv_from=2), None),
+        LayerSpec(T2, la(2, 2, 32, 32, 64, 24, 32, kv_from=2), None),
     ], side_dim=8, bigram_buckets=29, bigram_mul_prev=5, bigram_mul_cur=3, max_position=512)
     a, b, c = toks(200, 70), toks(90, 71), toks(40, 72)
 
