@@ -52,7 +52,7 @@ __global__ __launch_bounds__(1024) void latent_attn_rows_kernel(
     const T* __restrict__ cache, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens, int n_seqs, const int* __restrict__ positions, int H, int dim, int rd, int kr,
     int bs, float scale, int window, const float* __restrict__ cos_sin, int dims, int interleaved, T* __restrict__ out,
-    long long o_hs, long long o_ts, int DP, int DQ) {
+    long long o_hs, long long o_ts, int DP, int DQ, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int E = 16 / sizeof(T);
   constexpr int CE = VEC ? E : 1;                    // elements per value chunk
   constexpr int MAXC = VEC ? (sizeof(T) == 2 ? 2 : 4) : 8;
@@ -106,7 +106,12 @@ __global__ __launch_bounds__(1024) void latent_attn_rows_kernel(
     for (int j = 0; j < CE; ++j) o[c][j] = 0.f;
   const int nchunk = (kr + CE - 1) / CE;            // value chunks of the latent
 
-  for (int k0 = first; k0 <= pos; k0 += KT) {
+  // the row's key tiles, cut into gridDim.z contiguous runs (one workgroup each; a run may be empty)
+  const int ntiles = (pos - first + KT) / KT;
+  const int tps = (ntiles + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int t_hi = min(ntiles, ((int)blockIdx.z + 1) * tps);
+  for (int ti = blockIdx.z * tps; ti < t_hi; ++ti) {
+    const int k0 = first + ti * KT;
     const int n = min(KT, pos - k0 + 1);
     __syncthreads();                                 // the previous tile is fully read (and qs written)
     if constexpr (VEC) {
@@ -178,6 +183,24 @@ __global__ __launch_bounds__(1024) void latent_attn_rows_kernel(
     }
   }
   if (head_raw >= H) return;
+  if (part_o) {
+    // one of several runs: unnormalised sums and (max, sum of weights) for latent_attn_reduce_kernel
+    const size_t slot = ((size_t)blockIdx.z * H + head) * gridDim.x + row;
+    float* po = part_o + slot * kr;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int ci = lane + 64 * c;
+      if (ci < nchunk) {
+#pragma unroll
+        for (int j = 0; j < CE; ++j) po[(size_t)ci * CE + j] = o[c][j];
+      }
+    }
+    if (lane == 0) {
+      part_ml[2 * slot] = m_run;
+      part_ml[2 * slot + 1] = l_run;
+    }
+    return;
+  }
   const float inv = 1.f / l_run;
   T* op = out + (size_t)head * o_hs + (size_t)row * o_ts;
 #pragma unroll
@@ -187,6 +210,31 @@ __global__ __launch_bounds__(1024) void latent_attn_rows_kernel(
 #pragma unroll
       for (int j = 0; j < CE; ++j) stf<T>(op + (size_t)ci * CE + j, o[c][j] * inv);
     }
+  }
+}
+
+// out[h][row] = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M), M = max_z m_z; grid (rows, H), run 0 is never empty
+template <typename T>
+__global__ __launch_bounds__(256) void latent_attn_reduce_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml, int nsplit, int kr,
+                                                                 T* __restrict__ out, long long o_hs, long long o_ts) {
+  const int row = blockIdx.x, head = blockIdx.y, rows = gridDim.x, H = gridDim.y;
+  float M = -__builtin_inff();
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, part_ml[2 * (((size_t)z * H + head) * rows + row)]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const size_t slot = ((size_t)z * H + head) * rows + row;
+    L += part_ml[2 * slot + 1] * expf(part_ml[2 * slot] - M);
+  }
+  const float inv = 1.f / L;
+  T* op = out + (size_t)head * o_hs + (size_t)row * o_ts;
+  for (int e = threadIdx.x; e < kr; e += blockDim.x) {
+    float acc = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const size_t slot = ((size_t)z * H + head) * rows + row;
+      acc += part_o[slot * kr + e] * expf(part_ml[2 * slot] - M);
+    }
+    stf<T>(op + e, acc * inv);
   }
 }
 
@@ -211,7 +259,7 @@ template <typename T, bool VEC, int KT>
 int launch(const void* q, int q_stride, const void* q_lat, long long ql_hs, long long ql_ts, const void* cache,
            const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H,
            int dim, int rd, int kr, int bs, float scale, int window, const float* cos_sin, int dims, int interleaved,
-           void* out, long long o_hs, long long o_ts, int nw, hipStream_t s) {
+           void* out, long long o_hs, long long o_ts, int nw, int nsplit, float* part_o, float* part_ml, hipStream_t s) {
   constexpr int E = 16 / sizeof(T);
   const int D = kr + rd;
   const int DP = (D + E - 1) / E * E + E;           // padded row: 16-byte aligned, not a multiple of the bank span
@@ -227,10 +275,13 @@ int launch(const void* q, int q_stride, const void* q_lat, long long ql_hs, long
     allowed = allow_lds(latent_attn_rows_kernel<T, VEC, KT>, lds_max());
     if (allowed != 0) return allowed;
   }
-  const dim3 grid(rows, (H + nw - 1) / nw);
+  const dim3 grid(rows, (H + nw - 1) / nw, nsplit);
   latent_attn_rows_kernel<T, VEC, KT><<<grid, 64 * nw, lds, s>>>(
       (const T*)q, q_stride, (const T*)q_lat, ql_hs, ql_ts, (const T*)cache, block_tables, bt_stride, cu_seqlens, n_seqs,
-      positions, H, dim, rd, kr, bs, scale, window, cos_sin, dims, interleaved, (T*)out, o_hs, o_ts, DP, DQ);
+      positions, H, dim, rd, kr, bs, scale, window, cos_sin, dims, interleaved, (T*)out, o_hs, o_ts, DP, DQ,
+      nsplit > 1 ? part_o : nullptr, part_ml);
+  if (nsplit > 1)
+    latent_attn_reduce_kernel<T><<<dim3(rows, H), kr >= 256 ? 256 : 64, 0, s>>>(part_o, part_ml, nsplit, kr, (T*)out, o_hs, o_ts);
   return 0;
 }
 
@@ -238,15 +289,18 @@ int launch(const void* q, int q_stride, const void* q_lat, long long ql_hs, long
 
 // q [rows, H * (dim + rd)] (row stride q_stride); q_lat / out [H, rows, kr] with their own head and row strides;
 // cache [NB, 1, bs, kr + rd]; cu_seqlens (n_seqs + 1 row offsets) maps rows to block-table rows, nullptr: row i
-// uses table row i.  num_cus: workgroups are sized so that the grid covers the chip where the step allows.
+// uses table row i.  Workgroups are sized so that the grid covers the chip where the step allows; nsplit > 1 cuts
+// every row's keys into that many runs (steps of few rows over long contexts) whose partial results, in
+// part_o [nsplit, H, rows, kr] and part_ml [nsplit, H, rows, 2] (fp32), a second kernel combines.
 extern "C" int dgi_latent_attn_rows(const void* q, int q_stride, const void* q_lat, long long ql_hs, long long ql_ts,
                                     const void* cache, const int* block_tables, int bt_stride, const int* cu_seqlens,
                                     int n_seqs, const int* positions, int rows, int H, int dim, int rd, int kr,
                                     int block_size, float scale, int window, const float* cos_sin, int dims,
-                                    int interleaved, void* out, long long o_hs, long long o_ts, int is_f32,
-                                    hipStream_t s) {
+                                    int interleaved, void* out, long long o_hs, long long o_ts, int is_f32, int nsplit,
+                                    float* part_o, float* part_ml, hipStream_t s) {
   if (rows == 0) return 0;
   if (H <= 0 || kr <= 0 || rd < 0 || dim < 0 || window < 0) return -2;
+  if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (!part_o || !part_ml)) || H > 65535) return -7;
   if (dims > rd || (dims & 1) || (dims > 0 && !cos_sin)) return -3;
   if (H > 65535 * 16) return -4;
   const int E = is_f32 ? 4 : 8;
@@ -255,12 +309,12 @@ extern "C" int dgi_latent_attn_rows(const void* q, int q_stride, const void* q_l
   // heads per workgroup: as many as share a staged tile, fewer when the step has too few rows to fill the chip
   int nw = 16;
   while (nw > 1 && nw / 2 >= H) nw >>= 1;
-  while (nw > 2 && (long long)rows * ((H + nw - 1) / nw) < 512) nw >>= 1;
+  while (nw > 2 && (long long)rows * ((H + nw - 1) / nw) * nsplit < 512) nw >>= 1;
   int rc;
 #define DGI_LA(TT_, VV_, KK_)                                                                                       \
   rc = launch<TT_, VV_, KK_>(q, q_stride, q_lat, ql_hs, ql_ts, cache, block_tables, bt_stride, cu_seqlens, n_seqs, \
                              positions, rows, H, dim, rd, kr, block_size, scale, window, cos_sin, dims, interleaved, \
-                             out, o_hs, o_ts, nw, s)
+                             out, o_hs, o_ts, nw, nsplit, part_o, part_ml, s)
   if (is_f32) { if (vec) DGI_LA(float, true, 32); else DGI_LA(float, false, 32); }
   else { if (vec) DGI_LA(uint16_t, true, 64); else DGI_LA(uint16_t, false, 64); }
 #undef DGI_LA

@@ -262,7 +262,8 @@ class DepelixModel:
         o_lat = torch.empty(H, T, kr, device=q.device, dtype=q.dtype)
         if nd > 0:
             latent.latent_attn_rows(q[:nd], q_lat[:, :nd], cache, meta.dec_block_tables, None, meta.positions[:nd], H,
-                                    m.dim, m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter, out=o_lat[:, :nd])
+                                    m.dim, m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter, out=o_lat[:, :nd],
+                                    max_keys=meta.dec_block_tables.shape[1] * cache.shape[2])
         if meta.num_prefill_tokens > 0:
             latent.latent_attn_rows(q[nd:], q_lat[:, nd:], cache, meta.pre_block_tables, meta.pre_cu_seqlens,
                                     meta.positions[nd:], H, m.dim, m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter,
@@ -289,7 +290,8 @@ class DepelixModel:
             q_lat = torch.bmm(q[:nd].view(nd, H, m.qk_dim)[:, :, :m.dim].transpose(0, 1), L.uk)
             o_lat = torch.empty(H, nd, kr, device=q.device, dtype=q.dtype)
             latent.latent_attn_rows(q[:nd], q_lat, cache, meta.dec_block_tables, None, meta.positions[:nd], H, m.dim,
-                                    m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter, out=o_lat)
+                                    m.rot_dim, kr, m.scale, m.window, L.cos_sin, inter, out=o_lat,
+                                    max_keys=meta.dec_block_tables.shape[1] * cache.shape[2])
             latent.gate_heads(torch.bmm(o_lat, L.uv.transpose(1, 2)), None if gate is None else gate[:nd], per_head,
                               out=out[:nd])
         bt = meta.pre_block_tables

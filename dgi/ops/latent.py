@@ -21,6 +21,7 @@ missing), CPU tensors the ``*_ref`` function in fp32, which is also the kernel t
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional
 
 import torch
@@ -146,10 +147,22 @@ def latent_attn_rows_ref(o_lat, q, q_lat, cache, block_tables, cu_seqlens, posit
         o_lat[:, t] = (torch.softmax(s, dim=-1) @ rows[:, :kv_rank]).to(o_lat.dtype)
 
 
+SPLIT_WAVES = int(os.environ.get("DGI_LATENT_SPLIT_WAVES", "4096"))     # (row, head, run) waves a small step is cut into
+
+
+def split_runs(rows: int, heads: int, max_keys: int) -> int:
+    """Runs of keys per row for a step of ``rows`` x ``heads`` over at most ``max_keys`` keys: 1 when
+    the step fills the chip by itself or the bound is unknown, else enough for ``SPLIT_WAVES`` waves,
+    every run at least two 64-key tiles long, 16 at most."""
+    if max_keys <= 0 or rows <= 0 or rows * heads >= SPLIT_WAVES // 2:
+        return 1
+    return int(max(1, min(16, SPLIT_WAVES // (rows * heads), max_keys // 128)))
+
+
 def latent_attn_rows(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
                      cu_seqlens: Optional[torch.Tensor], positions: torch.Tensor, H: int, dim: int, rot_dim: int,
                      kv_rank: int, scale: float, window: int, cos_sin: Optional[torch.Tensor], interleaved: bool,
-                     out: torch.Tensor) -> torch.Tensor:
+                     out: torch.Tensor, max_keys: int = 0) -> torch.Tensor:
     """Softmax attention of every row over the cached rows ``[c | r]`` of its sequence
     (``cache`` [NB, 1, bs, kv_rank + rot_dim], pages by ``block_tables``; rows map to table rows
     through ``cu_seqlens``, None: row i <-> table row i).  Row t at position p sees keys
@@ -157,10 +170,18 @@ def latent_attn_rows(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, 
     ``(q_lat[h, t] . c_j + rot(q[t, h, dim:]) . r_j) * scale``: ``q_lat`` [H, T, kv_rank] is the
     unrotated query part folded through the key up-projection, ``q`` [T, H * (dim + rot_dim)] the
     query projection whose rotated part is rotated here by the row's position.  Writes the
-    weighted latent sums ``out`` [H, T, kv_rank] (any strides with unit inner stride)."""
+    weighted latent sums ``out`` [H, T, kv_rank] (any strides with unit inner stride).  ``max_keys``: an
+    upper bound of the keys a row sees, if the caller knows one — a step of few rows over many keys
+    is then cut into several runs of keys per row (more workgroups than rows x heads) and combined."""
     if _native(q):
+        T = q.shape[0]
+        nsplit = split_runs(T, H, min(max_keys, window) if window > 0 and max_keys > 0 else max_keys)
+        po = pm = None
+        if nsplit > 1:
+            po = torch.empty(nsplit * H * T * kv_rank, dtype=torch.float32, device=q.device)
+            pm = torch.empty(nsplit * H * T * 2, dtype=torch.float32, device=q.device)
         _call("latent_attn_rows", out, q, q_lat, cache, block_tables, cu_seqlens, positions, int(H), int(dim),
-              int(rot_dim), int(kv_rank), float(scale), int(window), cos_sin, bool(interleaved))
+              int(rot_dim), int(kv_rank), float(scale), int(window), cos_sin, bool(interleaved), nsplit, po, pm)
     else:
         latent_attn_rows_ref(out, q, q_lat, cache, block_tables, cu_seqlens, positions, H, dim, rot_dim, kv_rank, scale,
                              window, cos_sin, interleaved)

@@ -304,6 +304,12 @@ def test_latent_attention_rows_edges_and_far_keys(device, dtype, H, dim, rd, kr,
         want = torch.stack([attend_plain_folded(ql[:, i].cpu().to(F64), torch.stack([orc.rotate(qf[i, h, dim:], p, rd, 100.0, inter) for h in range(H)]),
                                                 cq, rq, window, scale, p) for i, p in enumerate(queries)], 1)
         close(out.float(), want, tol)
+    # few rows over many keys: every row's keys cut into runs (several workgroups per row and head), then combined
+    assert latent.split_runs(len(queries), H, N) > 1
+    out3 = torch.zeros(H, len(queries), kr, dtype=dtype, device=device)
+    latent.latent_attn_rows(q.to(device), ql, cache.to(device), tables, None, pos, H, dim, rd, kr, scale, window,
+                            cs.to(device), inter, out3, max_keys=N)
+    close(out3.float(), out.float(), 1e-5 if dtype == torch.float32 else 1e-2)
     # the same rows as portions of two sequences that share the pages (rows map to tables through cu_seqlens)
     order = sorted(range(len(queries)), key=lambda i: queries[i])
     idx = torch.tensor(order)
