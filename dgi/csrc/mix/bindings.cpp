@@ -69,7 +69,7 @@ int dgi_latent_attn_rows(const void* q, int q_stride, const void* q_lat, long lo
                          const void* cache, const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs,
                          const int* positions, int rows, int H, int dim, int rd, int kr, int block_size, float scale,
                          int window, const float* cos_sin, int dims, int interleaved, void* out, long long o_hs,
-                         long long o_ts, int is_f32, int nsplit, float* part_o, float* part_ml, hipStream_t s);
+                         long long o_ts, int is_f32, int nsplit, float* part_o, float* part_ml, int mfma, hipStream_t s);
 int dgi_glu_silu(void* out, const void* gu, int gu_stride, int rows, int I, int is_f32, hipStream_t s);
 int dgi_moe_expert_gate_up(float* mid, const void* h, int h_stride, const int* idx, const void* gate_up, int T, int E,
                            int top, int ff, int W, const float* pair_scale, int act, float limit, float alpha, int is_f32,
@@ -583,13 +583,15 @@ void latent_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& q_l
                       const at::Tensor& block_tables, const c10::optional<at::Tensor>& cu_seqlens, const at::Tensor& positions,
                       int64_t H, int64_t dim, int64_t rot_dim, int64_t kv_rank, double scale, int64_t window,
                       const c10::optional<at::Tensor>& cos_sin, bool interleaved, int64_t nsplit,
-                      c10::optional<at::Tensor> part_o, c10::optional<at::Tensor> part_ml) {
+                      c10::optional<at::Tensor> part_o, c10::optional<at::Tensor> part_ml, bool mfma) {
   const int f = act_kind(q, "q");
   float *pop = nullptr, *pmp = nullptr;
-  if (nsplit > 1) {
+  TORCH_CHECK(nsplit >= 1, "latent_attn_rows: nsplit >= 1");
+  const int64_t runs = nsplit;
+  if (runs > 1) {
     TORCH_CHECK(part_o.has_value() && part_ml.has_value(), "latent_attn_rows: split runs need their workspaces");
-    check_f32(*part_o, "part_o", nsplit * H * q.size(0) * kv_rank);
-    check_f32(*part_ml, "part_ml", nsplit * H * q.size(0) * 2);
+    check_f32(*part_o, "part_o", runs * H * q.size(0) * kv_rank);
+    check_f32(*part_ml, "part_ml", runs * H * q.size(0) * 2);
     pop = part_o->data_ptr<float>(); pmp = part_ml->data_ptr<float>();
   }
   check_rows(q, "q");
@@ -625,7 +627,7 @@ void latent_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& q_l
                                 (int)block_tables.stride(0), cu, n_seqs, i32p(positions, "positions", T), T, (int)H, (int)dim,
                                 (int)rot_dim, (int)kv_rank, (int)cache.size(2), (float)scale, (int)window, csp, dims,
                                 interleaved ? 1 : 0, out.data_ptr(), (long long)out.stride(0), (long long)out.stride(1), f,
-                                (int)std::max<int64_t>(1, nsplit), pop, pmp, cur_stream()), "latent_attn_rows");
+                                (int)nsplit, pop, pmp, mfma ? 1 : 0, cur_stream()), "latent_attn_rows");
 }
 
 void rotate_heads(at::Tensor x, const at::Tensor& positions, const at::Tensor& cos_sin, bool interleaved, int64_t H,
@@ -711,7 +713,7 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "Tensor positions, Tensor slots, Tensor? cos_sin, bool interleaved, Tensor(b!)? cache) -> ()");
   m.def("latent_attn_rows(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor cache, Tensor block_tables, Tensor? cu_seqlens, "
         "Tensor positions, int H, int dim, int rot_dim, int kv_rank, float scale, int window, Tensor? cos_sin, "
-        "bool interleaved, int nsplit=1, Tensor(b!)? part_o=None, Tensor(c!)? part_ml=None) -> ()");
+        "bool interleaved, int nsplit=1, Tensor(b!)? part_o=None, Tensor(c!)? part_ml=None, bool mfma=False) -> ()");
   m.def("rotate_heads(Tensor(a!) x, Tensor positions, Tensor cos_sin, bool interleaved, int H, int head_size, int offset) -> ()");
   m.def("gate_heads(Tensor(a!) out, Tensor ov, Tensor? gate, bool per_head) -> ()");
   m.def("gelu_tanh(Tensor(a!) out, Tensor x, Tensor? table, Tensor? ids, int col0) -> ()");

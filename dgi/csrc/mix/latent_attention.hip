@@ -21,6 +21,7 @@
 // result does not depend on how a prompt was cut into steps or on what else is in the batch.
 // The query's rotated part is rotated here, while it is staged (interleaved pairs or halves).
 // Scores, the online softmax and the accumulation are fp32; exp is the accurate expf.
+#include <algorithm>
 #include "../common.h"
 
 using namespace dgi;
@@ -238,6 +239,214 @@ __global__ __launch_bounds__(256) void latent_attn_reduce_kernel(const float* __
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// MFMA form (bf16; kr and kr + rd multiples of 16).  A workgroup owns one query row, a group of 16
+// heads and one run of the row's 64-key tiles; its four waves take 16 keys of every tile each and keep
+// their own running softmax, so nothing is exchanged between waves per tile.  Per tile and wave:
+//
+//   S^T [16 keys x 16 heads] = K [16 keys x D] Q^T [D x 16 heads]      D / 16 MFMAs 16x16x16; K rows from LDS,
+//                                                                     Q fragments held in registers
+//   O^T [kr x 16 heads]     += C^T [kr x 16 keys] P^T [16 keys x 16 heads]    kr / 16 MFMAs
+//
+// S^T comes out with a lane holding four consecutive keys of one head, which is exactly the operand
+// layout P^T needs, and O^T keeps a head's values in the lanes that hold its running maximum, so the
+// rescale needs no exchange either.  At the end the four waves' (max, sum, O^T) are combined in LDS and
+// the workgroup writes the row's result, or, when the row's keys are cut into gridDim.z runs, one
+// partial (max, sum, unnormalised O) per run for latent_attn_reduce_kernel.
+template <int NM, int NDS>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
+    const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ q_lat, long long ql_hs, long long ql_ts,
+    const uint16_t* __restrict__ cache, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ cu_seqlens, int n_seqs, const int* __restrict__ positions, int H, int dim, int rd, int kr,
+    int bs, float scale, int window, const float* __restrict__ cos_sin, int dims, int interleaved, int DP,
+    uint16_t* __restrict__ out, long long o_hs, long long o_ts, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int KT = 64;
+  extern __shared__ __attribute__((aligned(16))) uint16_t tile[];       // [KT][DP]; first holds the 16 queries
+  const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int D = kr + rd, nd = D >> 4, nm = kr >> 4;
+  const int row = blockIdx.x, rows = gridDim.x, g = blockIdx.y;
+
+  int seq = row;
+  if (cu_seqlens) {
+    int lo = 0, hi = n_seqs - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (cu_seqlens[mid] <= row) lo = mid; else hi = mid - 1;
+    }
+    seq = lo;
+  }
+  const int* bt = block_tables + (size_t)seq * bt_stride;
+  const int pos = positions[row];
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+
+  // the group's queries as bf16 rows [folded part | rotated part]; heads past H are zero rows
+  {
+    const int half = dims >> 1;
+    const float* cs = cos_sin ? cos_sin + (size_t)pos * dims : nullptr;
+    for (int i = threadIdx.x; i < 16 * D; i += 256) {
+      const int hh = i / D, e = i - hh * D;
+      const int head = g * 16 + hh;
+      uint16_t v = 0;
+      if (head < H) {
+        if (e < kr) {
+          v = q_lat[(size_t)head * ql_hs + (size_t)row * ql_ts + e];
+        } else {
+          const uint16_t* qr = q + (size_t)row * q_stride + (size_t)head * (dim + rd) + dim;
+          const int e2 = e - kr;
+          if (e2 < dims) {
+            int k, partner;
+            bool lead;                                  // the pair's first element
+            if (interleaved) { k = e2 >> 1; partner = e2 ^ 1; lead = !(e2 & 1); }
+            else { lead = e2 < half; k = lead ? e2 : e2 - half; partner = lead ? e2 + half : e2 - half; }
+            const float a = bf16_to_f32(qr[e2]), b = bf16_to_f32(qr[partner]);
+            const float c = cs[k], sn = cs[half + k];
+            v = f32_to_bf16(lead ? a * c - b * sn : a * c + b * sn);
+          } else {
+            v = qr[e2];
+          }
+        }
+      }
+      tile[(size_t)hh * DP + e] = v;
+    }
+  }
+  __syncthreads();
+  short4v qf[NDS];
+#pragma unroll
+  for (int s = 0; s < NDS; ++s) {
+    qf[s] = short4v{0, 0, 0, 0};
+    if (s < nd) qf[s] = *reinterpret_cast<const short4v*>(tile + (size_t)lr * DP + 16 * s + 4 * lg);
+  }
+
+  float m_run = -__builtin_inff(), l_run = 0.f;        // of head lr, over this wave's keys
+  f32x4 acc[NM];                                       // O^T: latent dims 16 m + 4 lg + i of head lr
+#pragma unroll
+  for (int m = 0; m < NM; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int ntiles = (pos - first + KT) / KT;
+  const int tps = (ntiles + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int t_hi = min(ntiles, ((int)blockIdx.z + 1) * tps);
+  const int cpr = D >> 3;                              // 16-byte chunks per cached row
+  for (int ti = blockIdx.z * tps; ti < t_hi; ++ti) {
+    const int k0 = first + ti * KT;
+    const int n = min(KT, pos - k0 + 1);
+    __syncthreads();                                   // the previous tile (or the queries) fully read
+    for (int i = threadIdx.x; i < KT * cpr; i += 256) {
+      const int j = i / cpr, c = i - j * cpr;
+      u32x4 v = {0u, 0u, 0u, 0u};                      // rows past the last key are zero: 0 * stale bits could be NaN
+      if (j < n) {
+        const int key = k0 + j;
+        const long long slot = (long long)bt[key / bs] * bs + (key % bs);
+        v = *reinterpret_cast<const u32x4*>(cache + slot * D + c * 8);
+      }
+      *reinterpret_cast<u32x4*>(tile + (size_t)j * DP + c * 8) = v;
+    }
+    __syncthreads();
+    if (16 * w >= n) continue;                         // none of this wave's 16 keys exists (wave-uniform)
+    f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+    const uint16_t* kp = tile + (size_t)(16 * w + lr) * DP + 4 * lg;
+#pragma unroll
+    for (int s = 0; s < NDS; ++s) {
+      if (s < nd) {
+        const short4v a = *reinterpret_cast<const short4v*>(kp + 16 * s);
+        sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sc, 0, 0, 0);
+      }
+    }
+    // sc[i]: key 16 w + 4 lg + i, head lr
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = (16 * w + 4 * lg + i < n) ? sc[i] * scale : -__builtin_inff();
+      mx = fmaxf(mx, sc[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));            // key 16 w exists: finite
+    const float m_new = fmaxf(m_run, mx);
+    const float corr = expf(m_run - m_new);            // first tile: exp(-inf) = 0
+    float p[4], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = expf(sc[i] - m_new);
+      sum += p[i];
+    }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    l_run = l_run * corr + sum;
+    m_run = m_new;
+    short4v pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pb[i] = (short)f32_to_bf16(p[i]);
+    const uint16_t* vp = tile + (size_t)(16 * w + 4 * lg) * DP + lr;
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      if (m < nm) {
+        short4v a;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = (short)vp[(size_t)j * DP + 16 * m];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[m][i] *= corr;
+        acc[m] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, acc[m], 0, 0, 0);
+      }
+    }
+  }
+  // combine the four waves: every head's (max, sum) through LDS, then O^T summed wave after wave in LDS
+  __syncthreads();                                     // the last tile is fully read
+  float* ml = reinterpret_cast<float*>(tile);          // [4 waves][16 heads][2], then [16 heads][2] combined
+  float* os = ml + 160;                                // [16 heads][kr + 4] fp32
+  const int ks = kr + 4;                               // padded: a head's rows start 4 banks apart
+  if (lg == 0) {
+    ml[(w * 16 + lr) * 2] = m_run;
+    ml[(w * 16 + lr) * 2 + 1] = l_run;
+  }
+  __syncthreads();
+  float M = -__builtin_inff();
+#pragma unroll
+  for (int ww = 0; ww < 4; ++ww) M = fmaxf(M, ml[(ww * 16 + lr) * 2]);
+  float Lsum = 0.f;
+#pragma unroll
+  for (int ww = 0; ww < 4; ++ww) {
+    const float mw = ml[(ww * 16 + lr) * 2];
+    Lsum += mw == -__builtin_inff() ? 0.f : ml[(ww * 16 + lr) * 2 + 1] * expf(mw - M);
+  }
+  const float f = m_run == -__builtin_inff() ? 0.f : expf(m_run - M);     // a wave (or a whole run) without keys adds nothing
+  for (int ww = 0; ww < 4; ++ww) {
+    if (w == ww) {
+#pragma unroll
+      for (int m = 0; m < NM; ++m) {
+        if (m < nm) {
+          float4* dst = reinterpret_cast<float4*>(os + (size_t)lr * ks + 16 * m + 4 * lg);
+          float4 cur = ww == 0 ? make_float4(0.f, 0.f, 0.f, 0.f) : *dst;
+          cur.x += acc[m][0] * f; cur.y += acc[m][1] * f; cur.z += acc[m][2] * f; cur.w += acc[m][3] * f;
+          *dst = cur;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (w == 0 && lg == 0) {                             // every wave has read the per-wave entries before the barriers above
+    ml[128 + lr * 2] = M;
+    ml[128 + lr * 2 + 1] = Lsum;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 16 * kr; i += 256) {
+    const int hh = i / kr, e = i - hh * kr;
+    const int head = g * 16 + hh;
+    if (head >= H) break;
+    const float v = os[(size_t)hh * ks + e];
+    if (part_o) {
+      const size_t slot = ((size_t)blockIdx.z * H + head) * rows + row;
+      part_o[slot * kr + e] = v;
+      if (e == 0) {
+        part_ml[2 * slot] = ml[128 + hh * 2];
+        part_ml[2 * slot + 1] = ml[128 + hh * 2 + 1];
+      }
+    } else {
+      out[(size_t)head * o_hs + (size_t)row * o_ts + e] = f32_to_bf16(v / ml[128 + hh * 2 + 1]);
+    }
+  }
+}
+
 template <typename K>
 int allow_lds(K kernel, size_t lds) {
   return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -285,6 +494,32 @@ int launch(const void* q, int q_stride, const void* q_lat, long long ql_hs, long
   return 0;
 }
 
+
+template <int NM, int NDS>
+int launch_mfma(const void* q, int q_stride, const void* q_lat, long long ql_hs, long long ql_ts, const void* cache,
+                const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows,
+                int H, int dim, int rd, int kr, int bs, float scale, int window, const float* cos_sin, int dims,
+                int interleaved, void* out, long long o_hs, long long o_ts, int nsplit, float* part_o, float* part_ml,
+                hipStream_t s) {
+  const int D = kr + rd;
+  const int DP = D + 8;                                // rows 16-byte aligned, consecutive rows 4 banks apart
+  const size_t lds = std::max((size_t)64 * DP * 2, (size_t)(160 + 16 * (kr + 4)) * 4);     // tiles, then the combine buffers
+  if (lds > lds_max()) return -6;
+  static int allowed = -1;
+  if (allowed != 0 && lds > 64 * 1024) {
+    allowed = allow_lds(latent_attn_mfma_kernel<NM, NDS>, lds_max());
+    if (allowed != 0) return allowed;
+  }
+  latent_attn_mfma_kernel<NM, NDS><<<dim3(rows, (H + 15) / 16, nsplit), 256, lds, s>>>(
+      (const uint16_t*)q, q_stride, (const uint16_t*)q_lat, ql_hs, ql_ts, (const uint16_t*)cache, block_tables, bt_stride,
+      cu_seqlens, n_seqs, positions, H, dim, rd, kr, bs, scale, window, cos_sin, dims, interleaved, DP, (uint16_t*)out, o_hs,
+      o_ts, nsplit > 1 ? part_o : nullptr, part_ml);
+  if (nsplit > 1)
+    latent_attn_reduce_kernel<uint16_t><<<dim3(rows, H), kr >= 256 ? 256 : 64, 0, s>>>(part_o, part_ml, nsplit, kr,
+                                                                                      (uint16_t*)out, o_hs, o_ts);
+  return 0;
+}
+
 }  // namespace
 
 // q [rows, H * (dim + rd)] (row stride q_stride); q_lat / out [H, rows, kr] with their own head and row strides;
@@ -297,10 +532,26 @@ extern "C" int dgi_latent_attn_rows(const void* q, int q_stride, const void* q_l
                                     int n_seqs, const int* positions, int rows, int H, int dim, int rd, int kr,
                                     int block_size, float scale, int window, const float* cos_sin, int dims,
                                     int interleaved, void* out, long long o_hs, long long o_ts, int is_f32, int nsplit,
-                                    float* part_o, float* part_ml, hipStream_t s) {
+                                    float* part_o, float* part_ml, int mfma, hipStream_t s) {
   if (rows == 0) return 0;
   if (H <= 0 || kr <= 0 || rd < 0 || dim < 0 || window < 0) return -2;
   if (nsplit < 1 || nsplit > 65535 || (nsplit > 1 && (!part_o || !part_ml)) || H > 65535) return -7;
+  if (mfma) {
+    if (is_f32 || kr % 16 || (kr + rd) % 16 || kr > 512 || kr + rd > 576 || ((uintptr_t)cache & 15)) return -8;
+    if (dims > rd || (dims & 1) || (dims > 0 && !cos_sin)) return -3;
+    int rc;
+    if (kr <= 128 && kr + rd <= 192)
+      rc = launch_mfma<8, 12>(q, q_stride, q_lat, ql_hs, ql_ts, cache, block_tables, bt_stride, cu_seqlens, n_seqs, positions,
+                              rows, H, dim, rd, kr, block_size, scale, window, cos_sin, dims, interleaved, out, o_hs, o_ts,
+                              nsplit, part_o, part_ml, s);
+    else
+      rc = launch_mfma<32, 36>(q, q_stride, q_lat, ql_hs, ql_ts, cache, block_tables, bt_stride, cu_seqlens, n_seqs, positions,
+                               rows, H, dim, rd, kr, block_size, scale, window, cos_sin, dims, interleaved, out, o_hs, o_ts,
+                               nsplit, part_o, part_ml, s);
+    if (rc != 0) return rc;
+    DGI_CHECK_LAUNCH();
+    return 0;
+  }
   if (dims > rd || (dims & 1) || (dims > 0 && !cos_sin)) return -3;
   if (H > 65535 * 16) return -4;
   const int E = is_f32 ? 4 : 8;

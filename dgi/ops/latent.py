@@ -150,6 +150,16 @@ def latent_attn_rows_ref(o_lat, q, q_lat, cache, block_tables, cu_seqlens, posit
 SPLIT_WAVES = int(os.environ.get("DGI_LATENT_SPLIT_WAVES", "4096"))     # (row, head, run) waves a small step is cut into
 
 
+MFMA_ROWS = os.environ.get("DGI_LATENT_MFMA", "1") == "1"     # 0: bf16 rows on the element-wise kernel too (A/B)
+
+
+def mfma_rows_ok(dtype, kv_rank: int, rot_dim: int) -> bool:
+    """Whether ``latent_attn_rows`` takes its MFMA kernel: bf16, latent and latent + key part multiples
+    of 16, at most 512 / 576 wide (accumulators and query fragments live in registers)."""
+    return (MFMA_ROWS and dtype == torch.bfloat16 and kv_rank % 16 == 0 and (kv_rank + rot_dim) % 16 == 0
+            and kv_rank <= 512 and kv_rank + rot_dim <= 576)
+
+
 def split_runs(rows: int, heads: int, max_keys: int) -> int:
     """Runs of keys per row for a step of ``rows`` x ``heads`` over at most ``max_keys`` keys: 1 when
     the step fills the chip by itself or the bound is unknown, else enough for ``SPLIT_WAVES`` waves,
@@ -175,13 +185,15 @@ def latent_attn_rows(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, 
     is then cut into several runs of keys per row (more workgroups than rows x heads) and combined."""
     if _native(q):
         T = q.shape[0]
-        nsplit = split_runs(T, H, min(max_keys, window) if window > 0 and max_keys > 0 else max_keys)
+        mfma = mfma_rows_ok(q.dtype, kv_rank, rot_dim)
+        nsplit = split_runs(T, (H + 15) // 16 * 4 if mfma else H,
+                            min(max_keys, window) if window > 0 and max_keys > 0 else max_keys)
         po = pm = None
         if nsplit > 1:
             po = torch.empty(nsplit * H * T * kv_rank, dtype=torch.float32, device=q.device)
             pm = torch.empty(nsplit * H * T * 2, dtype=torch.float32, device=q.device)
         _call("latent_attn_rows", out, q, q_lat, cache, block_tables, cu_seqlens, positions, int(H), int(dim),
-              int(rot_dim), int(kv_rank), float(scale), int(window), cos_sin, bool(interleaved), nsplit, po, pm)
+              int(rot_dim), int(kv_rank), float(scale), int(window), cos_sin, bool(interleaved), nsplit, po, pm, mfma)
     else:
         latent_attn_rows_ref(out, q, q_lat, cache, block_tables, cu_seqlens, positions, H, dim, rot_dim, kv_rank, scale,
                              window, cos_sin, interleaved)

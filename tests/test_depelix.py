@@ -253,7 +253,8 @@ def attend_plain(qn, qr, c, r, uk, window, scale, p):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,dim,rd,kr,window,inter", [(3, 8, 4, 12, 5, False), (2, 4, 6, 8, 0, True), (5, 6, 2, 9, 17, False),
-                                                      (6, 16, 8, 24, 64, True), (17, 8, 8, 64, 33, False)])
+                                                      (6, 16, 8, 24, 64, True), (17, 8, 8, 64, 33, False),
+                                                      (4, 16, 16, 32, 70, False), (19, 8, 32, 64, 0, True), (16, 24, 16, 144, 129, True)])
 def test_latent_attention_rows_edges_and_far_keys(device, dtype, H, dim, rd, kr, window, inter):
     """Decode rows and prompt rows over scattered pages.  One key is made to dominate a head's scores (its
     latent is a large multiple of the folded query) and placed just inside the window, just outside it, at
