@@ -260,7 +260,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     const uint16_t* __restrict__ cache, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_seqlens, int n_seqs, const int* __restrict__ positions, int H, int dim, int rd, int kr,
     int bs, float scale, int window, const float* __restrict__ cos_sin, int dims, int interleaved, int DP,
-    uint16_t* __restrict__ out, long long o_hs, long long o_ts, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    uint16_t* __restrict__ out, long long o_hs, long long o_ts, float* __restrict__ part_o, float* __restrict__ part_ml,
+    unsigned cpr_magic) {
   constexpr int KT = 64;
   extern __shared__ __attribute__((aligned(16))) uint16_t tile[];       // [KT][DP]; first holds the 16 queries
   const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -285,30 +286,50 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   {
     const int half = dims >> 1;
     const float* cs = cos_sin ? cos_sin + (size_t)pos * dims : nullptr;
-    for (int i = threadIdx.x; i < 16 * D; i += 256) {
-      const int hh = i / D, e = i - hh * D;
+    // folded part: 16-byte copies where the query tensor allows them (all issued before any lands)
+    const bool qvec = ((uintptr_t)q_lat & 15) == 0 && (ql_hs & 7) == 0 && (ql_ts & 7) == 0;
+    if (qvec) {
+      constexpr int NQ = (16 * NM * 2 + 255) / 256;
+      const int cq = kr >> 3;
+#pragma unroll
+      for (int it = 0; it < NQ; ++it) {
+        const int idx = threadIdx.x + 256 * it;
+        const int hh = idx / cq, c = idx - hh * cq;
+        if (hh < 16) {
+          const int head = g * 16 + hh;
+          u32x4 v = {0u, 0u, 0u, 0u};
+          if (head < H) v = *reinterpret_cast<const u32x4*>(q_lat + (size_t)head * ql_hs + (size_t)row * ql_ts + c * 8);
+          *reinterpret_cast<u32x4*>(tile + (size_t)hh * DP + c * 8) = v;
+        }
+      }
+    } else {
+      for (int i = threadIdx.x; i < 16 * kr; i += 256) {
+        const int hh = i / kr, e = i - hh * kr;
+        const int head = g * 16 + hh;
+        tile[(size_t)hh * DP + e] = head < H ? q_lat[(size_t)head * ql_hs + (size_t)row * ql_ts + e] : (uint16_t)0;
+      }
+    }
+    // rotated part
+#pragma unroll 4
+    for (int i = threadIdx.x; i < 16 * rd; i += 256) {
+      const int hh = i / rd, e2 = i - hh * rd;
       const int head = g * 16 + hh;
       uint16_t v = 0;
       if (head < H) {
-        if (e < kr) {
-          v = q_lat[(size_t)head * ql_hs + (size_t)row * ql_ts + e];
+        const uint16_t* qr = q + (size_t)row * q_stride + (size_t)head * (dim + rd) + dim;
+        if (e2 < dims) {
+          int k, partner;
+          bool lead;                                  // the pair's first element
+          if (interleaved) { k = e2 >> 1; partner = e2 ^ 1; lead = !(e2 & 1); }
+          else { lead = e2 < half; k = lead ? e2 : e2 - half; partner = lead ? e2 + half : e2 - half; }
+          const float a = bf16_to_f32(qr[e2]), b = bf16_to_f32(qr[partner]);
+          const float c = cs[k], sn = cs[half + k];
+          v = f32_to_bf16(lead ? a * c - b * sn : a * c + b * sn);
         } else {
-          const uint16_t* qr = q + (size_t)row * q_stride + (size_t)head * (dim + rd) + dim;
-          const int e2 = e - kr;
-          if (e2 < dims) {
-            int k, partner;
-            bool lead;                                  // the pair's first element
-            if (interleaved) { k = e2 >> 1; partner = e2 ^ 1; lead = !(e2 & 1); }
-            else { lead = e2 < half; k = lead ? e2 : e2 - half; partner = lead ? e2 + half : e2 - half; }
-            const float a = bf16_to_f32(qr[e2]), b = bf16_to_f32(qr[partner]);
-            const float c = cs[k], sn = cs[half + k];
-            v = f32_to_bf16(lead ? a * c - b * sn : a * c + b * sn);
-          } else {
-            v = qr[e2];
-          }
+          v = qr[e2];
         }
       }
-      tile[(size_t)hh * DP + e] = v;
+      tile[(size_t)hh * DP + kr + e2] = v;
     }
   }
   __syncthreads();
@@ -328,31 +349,59 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   const int tps = (ntiles + (int)gridDim.z - 1) / (int)gridDim.z;
   const int t_hi = min(ntiles, ((int)blockIdx.z + 1) * tps);
   const int cpr = D >> 3;                              // 16-byte chunks per cached row
-  for (int ti = blockIdx.z * tps; ti < t_hi; ++ti) {
+  // A wave stages only its own 16 rows of a tile (nobody else reads them), so the waves run their tiles
+  // without workgroup barriers, and the rows of tile t + 1 are loaded into registers before tile t is
+  // computed: the loads' latency hides behind the MFMAs.
+  constexpr int NLD = (16 * NDS * 2 + 63) / 64;        // 16-byte chunks per lane: 16 rows of at most NDS * 2 chunks
+  u32x4 pre[NLD];
+  auto issue = [&](int ti) {
+    const int k0 = first + ti * KT + 16 * w;
+    // lane j < 16 resolves the cache slot of the wave's row j once; the chunk loads fetch it by shuffle
+    int myslot = -1;                                   // rows past the last key: none
+    if (lane < 16 && k0 + lane <= pos) {
+      const int key = k0 + lane;
+      myslot = bt[key / bs] * bs + (key % bs);
+    }
+#pragma unroll
+    for (int it = 0; it < NLD; ++it) {
+      const int idx = lane + 64 * it;
+      const int j = (int)__umulhi((unsigned)idx, cpr_magic), c = idx - j * cpr;     // idx / cpr (checked on the host)
+      const int sl = __shfl(myslot, j & 15, 64);
+      pre[it] = u32x4{0u, 0u, 0u, 0u};                 // rows past the last key are zero: 0 * stale bits could be NaN
+      if (j < 16 && sl >= 0) pre[it] = *reinterpret_cast<const u32x4*>(cache + (long long)sl * D + c * 8);
+    }
+  };
+  const int t_lo = blockIdx.z * tps;
+  __syncthreads();                                     // every wave has its query fragments: the tile region is free
+  if (t_lo < t_hi) issue(t_lo);
+  for (int ti = t_lo; ti < t_hi; ++ti) {
     const int k0 = first + ti * KT;
     const int n = min(KT, pos - k0 + 1);
-    __syncthreads();                                   // the previous tile (or the queries) fully read
-    for (int i = threadIdx.x; i < KT * cpr; i += 256) {
-      const int j = i / cpr, c = i - j * cpr;
-      u32x4 v = {0u, 0u, 0u, 0u};                      // rows past the last key are zero: 0 * stale bits could be NaN
-      if (j < n) {
-        const int key = k0 + j;
-        const long long slot = (long long)bt[key / bs] * bs + (key % bs);
-        v = *reinterpret_cast<const u32x4*>(cache + slot * D + c * 8);
-      }
-      *reinterpret_cast<u32x4*>(tile + (size_t)j * DP + c * 8) = v;
+#pragma unroll
+    for (int it = 0; it < NLD; ++it) {
+      const int idx = lane + 64 * it;
+      const int j = (int)__umulhi((unsigned)idx, cpr_magic), c = idx - j * cpr;
+      if (j < 16) *reinterpret_cast<u32x4*>(tile + (size_t)(16 * w + j) * DP + c * 8) = pre[it];
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (ti + 1 < t_hi) issue(ti + 1);
     if (16 * w >= n) continue;                         // none of this wave's 16 keys exists (wave-uniform)
-    f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+    // four independent accumulation chains (a chain of dependent MFMAs waits out each one's latency)
+    f32x4 sp[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) sp[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     const uint16_t* kp = tile + (size_t)(16 * w + lr) * DP + 4 * lg;
 #pragma unroll
     for (int s = 0; s < NDS; ++s) {
       if (s < nd) {
         const short4v a = *reinterpret_cast<const short4v*>(kp + 16 * s);
-        sc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sc, 0, 0, 0);
+        sp[s & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sp[s & 3], 0, 0, 0);
       }
     }
+    f32x4 sc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sc[i] = (sp[0][i] + sp[1][i]) + (sp[2][i] + sp[3][i]);
     // sc[i]: key 16 w + 4 lg + i, head lr
     float mx = -__builtin_inff();
 #pragma unroll
@@ -377,6 +426,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     short4v pb;
 #pragma unroll
     for (int i = 0; i < 4; ++i) pb[i] = (short)f32_to_bf16(p[i]);
+    const bool rescale = __any(corr != 1.f);           // no head's maximum moved: the sums keep their scale
     const uint16_t* vp = tile + (size_t)(16 * w + 4 * lg) * DP + lr;
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
@@ -384,11 +434,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
         short4v a;
 #pragma unroll
         for (int j = 0; j < 4; ++j) a[j] = (short)vp[(size_t)j * DP + 16 * m];
+        if (rescale) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[m][i] *= corr;
+          for (int i = 0; i < 4; ++i) acc[m][i] *= corr;
+        }
         acc[m] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, acc[m], 0, 0, 0);
       }
     }
+    __builtin_amdgcn_wave_barrier();                   // this tile's rows are read before the next ones land
   }
   // combine the four waves: every head's (max, sum) through LDS, then O^T summed wave after wave in LDS
   __syncthreads();                                     // the last tile is fully read
@@ -503,6 +556,11 @@ int launch_mfma(const void* q, int q_stride, const void* q_lat, long long ql_hs,
                 hipStream_t s) {
   const int D = kr + rd;
   const int DP = D + 8;                                // rows 16-byte aligned, consecutive rows 4 banks apart
+  // idx / cpr for idx < 16 * cpr + 64 as a multiply-high (cpr = 16-byte chunks per cached row)
+  const unsigned cpr = (unsigned)D >> 3;
+  const unsigned magic = (unsigned)((0x100000000ull + cpr - 1) / cpr);
+  for (unsigned i = 0; i < 16 * cpr + 64; ++i)
+    if ((unsigned)(((unsigned long long)i * magic) >> 32) != i / cpr) return -9;
   const size_t lds = std::max((size_t)64 * DP * 2, (size_t)(160 + 16 * (kr + 4)) * 4);     // tiles, then the combine buffers
   if (lds > lds_max()) return -6;
   static int allowed = -1;
@@ -513,7 +571,7 @@ int launch_mfma(const void* q, int q_stride, const void* q_lat, long long ql_hs,
   latent_attn_mfma_kernel<NM, NDS><<<dim3(rows, (H + 15) / 16, nsplit), 256, lds, s>>>(
       (const uint16_t*)q, q_stride, (const uint16_t*)q_lat, ql_hs, ql_ts, (const uint16_t*)cache, block_tables, bt_stride,
       cu_seqlens, n_seqs, positions, H, dim, rd, kr, bs, scale, window, cos_sin, dims, interleaved, DP, (uint16_t*)out, o_hs,
-      o_ts, nsplit > 1 ? part_o : nullptr, part_ml);
+      o_ts, nsplit > 1 ? part_o : nullptr, part_ml, magic);
   if (nsplit > 1)
     latent_attn_reduce_kernel<uint16_t><<<dim3(rows, H), kr >= 256 ? 256 : 64, 0, s>>>(part_o, part_ml, nsplit, kr,
                                                                                       (uint16_t*)out, o_hs, o_ts);

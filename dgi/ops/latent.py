@@ -186,7 +186,8 @@ def latent_attn_rows(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, 
     if _native(q):
         T = q.shape[0]
         mfma = mfma_rows_ok(q.dtype, kv_rank, rot_dim)
-        nsplit = split_runs(T, (H + 15) // 16 * 4 if mfma else H,
+        # the MFMA kernel's workgroups (16 heads, 4 waves) are best at about one per compute unit
+        nsplit = split_runs(T, (H + 15) // 16 * 16 if mfma else H,
                             min(max_keys, window) if window > 0 and max_keys > 0 else max_keys)
         po = pm = None
         if nsplit > 1:

@@ -311,6 +311,13 @@ def test_latent_attention_rows_edges_and_far_keys(device, dtype, H, dim, rd, kr,
     latent.latent_attn_rows(q.to(device), ql, cache.to(device), tables, None, pos, H, dim, rd, kr, scale, window,
                             cs.to(device), inter, out3, max_keys=N)
     close(out3.float(), out.float(), 1e-5 if dtype == torch.float32 else 1e-2)
+    # a folded query that sits at an odd offset inside a wider buffer (no 16-byte accesses possible)
+    wide = torch.zeros(H, len(queries), kr + 6, dtype=dtype, device=device)
+    wide[:, :, 3:kr + 3] = ql
+    out4 = torch.zeros(H, len(queries), kr, dtype=dtype, device=device)
+    latent.latent_attn_rows(q.to(device), wide[:, :, 3:kr + 3], cache.to(device), tables, None, pos, H, dim, rd, kr, scale,
+                            window, cs.to(device), inter, out4)
+    close(out4.float(), out.float(), 1e-5 if dtype == torch.float32 else 1e-2)
     # the same rows as portions of two sequences that share the pages (rows map to tables through cu_seqlens)
     order = sorted(range(len(queries)), key=lambda i: queries[i])
     idx = torch.tensor(order)
