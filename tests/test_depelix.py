@@ -690,3 +690,17 @@ def test_mfma_prompt_path_in_the_model(monkeypatch):
     slow = run()
     assert len(calls) == 8
     close(fast, slow, 0.06 * max(1.0, slow.abs().max().item()))
+
+
+def test_worker_engine_serves_a_checkpoint_dir(tmp_path):
+    """The worker's native engine picks the model class from config.json and generates through the same LLMEngine."""
+    sys.path.insert(0, os.path.join(ROOT, "worker"))
+    from engines.llm_native import NativeLLMEngine
+    d = str(tmp_path / "ckpt")
+    write_checkpoint(engine(small_cfg(vocab_size=300), "cpu", torch.bfloat16), d)
+    e = NativeLLMEngine({"model_id": d, "device": "cpu", "max_model_len": 128, "max_num_batched_tokens": 128,
+                         "num_blocks": 64, "max_num_seqs": 4})
+    e.load_model()
+    assert type(e.engine.model).__name__ == "DepelixModel"
+    out = e.batch_inference([{"messages": [{"role": "user", "content": "hi"}], "max_tokens": 5, "temperature": 0.0}])
+    assert out[0]["usage"]["completion_tokens"] == 5
