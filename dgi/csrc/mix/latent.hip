@@ -131,7 +131,7 @@ __global__ __launch_bounds__(NT) void stream_add_norm_kernel(float* __restrict__
 
 // One workgroup per row.  Query latent: columns [0, q_rank); key/value latent [q_rank, q_rank + kv_rank);
 // key part [q_rank + kv_rank, q_rank + kv_rank + rot_dim), of which the first `dims` rotate.
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(NT) void latent_prep_kernel(const T* __restrict__ proj, int stride, int q_rank, int kv_rank,
                                                          int rot_dim, const float* __restrict__ dq_w,
                                                          const float* __restrict__ dkv_w, float eps,
@@ -141,28 +141,53 @@ __global__ __launch_bounds__(NT) void latent_prep_kernel(const T* __restrict__ p
   __shared__ float red[NT / 64];
   const int row = blockIdx.x;
   const T* p = proj + (size_t)row * stride;
-  {
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < q_rank; c += NT) {
-      const float v = ldf<T>(p + c);
-      ss += v * v;
+  // RMS norm of n values at src times w -> dst; VEC: 16-byte chunks held in registers between the sum and the store
+  auto norm_part = [&](const T* src, int n, const float* w, T* dst) {
+    constexpr int E = 16 / sizeof(T);
+    if (VEC) {
+      float v[2][8];
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int c = (threadIdx.x + k * NT) * E;
+        if (c < n) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(src + c);
+          if constexpr (sizeof(T) == 2) unpack8(__builtin_bit_cast(u32x4, raw), v[k]);
+          else { v[k][0] = __uint_as_float(raw.x); v[k][1] = __uint_as_float(raw.y); v[k][2] = __uint_as_float(raw.z); v[k][3] = __uint_as_float(raw.w); }
+#pragma unroll
+          for (int j = 0; j < E; ++j) ss += v[k][j] * v[k][j];
+        }
+      }
+      const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int c = (threadIdx.x + k * NT) * E;
+        if (c < n) {
+#pragma unroll
+          for (int j = 0; j < E; ++j) v[k][j] *= inv * w[c + j];
+          uint4 o;
+          if constexpr (sizeof(T) == 2) o = __builtin_bit_cast(uint4, pack8(v[k]));
+          else o = make_uint4(__float_as_uint(v[k][0]), __float_as_uint(v[k][1]), __float_as_uint(v[k][2]), __float_as_uint(v[k][3]));
+          *reinterpret_cast<uint4*>(dst + c) = o;
+        }
+      }
+    } else {
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < n; c += NT) {
+        const float x = ldf<T>(src + c);
+        ss += x * x;
+      }
+      const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+      for (int c = threadIdx.x; c < n; c += NT) stf<T>(dst + c, ldf<T>(src + c) * inv * w[c]);
     }
-    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)q_rank + eps);
-    T* o = cq + (size_t)row * q_rank;
-    for (int c = threadIdx.x; c < q_rank; c += NT) stf<T>(o + c, ldf<T>(p + c) * inv * dq_w[c]);
-  }
+  };
+  norm_part(p, q_rank, dq_w, cq + (size_t)row * q_rank);
   if (!cache) return;
   const int slot = slots[row];
   if (slot < 0) return;                               // uniform over the workgroup
   T* dst = cache + (size_t)slot * (kv_rank + rot_dim);
   const T* lat = p + q_rank;
-  float ss = 0.f;
-  for (int c = threadIdx.x; c < kv_rank; c += NT) {
-    const float v = ldf<T>(lat + c);
-    ss += v * v;
-  }
-  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)kv_rank + eps);
-  for (int c = threadIdx.x; c < kv_rank; c += NT) stf<T>(dst + c, ldf<T>(lat + c) * inv * dkv_w[c]);
+  norm_part(lat, kv_rank, dkv_w, dst);
   const T* kp = lat + kv_rank;
   T* kd = dst + kv_rank;
   const int half = dims >> 1;
@@ -210,8 +235,45 @@ __global__ __launch_bounds__(NT) void gate_heads_kernel(T* __restrict__ out, con
   stf<T>(out + (size_t)t * H * dv + c, v);
 }
 
+// tanh(a) = sign(a) (1 - e) / (1 + e), e = exp(-2 |a|), through the hardware exp / rcp (absolute error below 2e-7)
+// eight (bf16) / four (fp32) consecutive value dims per thread: dv, the strides and the pointers allow 16-byte accesses
+template <typename T>
+__global__ __launch_bounds__(NT) void gate_heads_vec_kernel(T* __restrict__ out, const T* __restrict__ ov, long long ov_hs,
+                                                            long long ov_ts, const T* __restrict__ gate, int gate_stride,
+                                                            int per_head, int H, int dv) {
+  constexpr int E = 16 / sizeof(T);
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * NT + threadIdx.x) * E;
+  if (c >= H * dv) return;
+  const int h = c / dv, d = c - h * dv;
+  const uint4 raw = *reinterpret_cast<const uint4*>(ov + (size_t)h * ov_hs + (size_t)t * ov_ts + d);
+  float v[8], g[8];
+  if constexpr (sizeof(T) == 2) unpack8(__builtin_bit_cast(u32x4, raw), v);
+  else { v[0] = __uint_as_float(raw.x); v[1] = __uint_as_float(raw.y); v[2] = __uint_as_float(raw.z); v[3] = __uint_as_float(raw.w); }
+  if (gate) {
+    if (per_head) {
+      const float s = 1.f / (1.f + expf(-ldf<T>(gate + (size_t)t * gate_stride + h)));
+#pragma unroll
+      for (int j = 0; j < E; ++j) v[j] *= s;
+    } else {
+      const uint4 gr = *reinterpret_cast<const uint4*>(gate + (size_t)t * gate_stride + c);
+      if constexpr (sizeof(T) == 2) unpack8(__builtin_bit_cast(u32x4, gr), g);
+      else { g[0] = __uint_as_float(gr.x); g[1] = __uint_as_float(gr.y); g[2] = __uint_as_float(gr.z); g[3] = __uint_as_float(gr.w); }
+#pragma unroll
+      for (int j = 0; j < E; ++j) v[j] *= 1.f / (1.f + expf(-g[j]));
+    }
+  }
+  uint4 o;
+  if constexpr (sizeof(T) == 2) o = __builtin_bit_cast(uint4, pack8(v));
+  else o = make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3]));
+  *reinterpret_cast<uint4*>(out + (size_t)t * H * dv + c) = o;
+}
+
 __device__ __forceinline__ float gelu_tanh_f(float z) {
-  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  const float a = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  const float e = __expf(-2.f * fabsf(a));
+  const float t = copysignf((1.f - e) * __builtin_amdgcn_rcpf(1.f + e), a);
+  return 0.5f * z * (1.f + t);
 }
 
 // out[t][c] = gelu(x[t][c]) (* table[ids[t]][col0 + c]); grid-stride over T * n
@@ -275,13 +337,16 @@ extern "C" int dgi_latent_prep(const void* proj, int stride, int is_f32, int T, 
   if (q_rank <= 0) return -2;
   if (cache && (kv_rank <= 0 || rot_dim < 0 || dims > rot_dim || (dims & 1) || (dims > 0 && !cos_sin) || !dkv_w || !slots))
     return -3;
-  if (is_f32)
-    latent_prep_kernel<float><<<T, NT, 0, s>>>((const float*)proj, stride, q_rank, kv_rank, rot_dim, dq_w, dkv_w, eps,
-                                               positions, slots, cos_sin, dims, interleaved, (float*)cq, (float*)cache);
-  else
-    latent_prep_kernel<uint16_t><<<T, NT, 0, s>>>((const uint16_t*)proj, stride, q_rank, kv_rank, rot_dim, dq_w, dkv_w, eps,
-                                                  positions, slots, cos_sin, dims, interleaved, (uint16_t*)cq,
-                                                  (uint16_t*)cache);
+  // 16-byte accesses: both latents and every row / cache start are multiples of the chunk, at most two chunks a thread
+  const int E = is_f32 ? 4 : 8;
+  const bool vec = q_rank % E == 0 && stride % E == 0 && q_rank <= 2 * NT * E && (((uintptr_t)proj | (uintptr_t)cq) & 15) == 0 &&
+                   (!cache || (kv_rank % E == 0 && (kv_rank + rot_dim) % E == 0 && kv_rank <= 2 * NT * E && ((uintptr_t)cache & 15) == 0));
+#define DGI_LP(TT_, VV_)                                                                                                  \
+  latent_prep_kernel<TT_, VV_><<<T, NT, 0, s>>>((const TT_*)proj, stride, q_rank, kv_rank, rot_dim, dq_w, dkv_w, eps, positions, \
+                                               slots, cos_sin, dims, interleaved, (TT_*)cq, (TT_*)cache)
+  if (is_f32) { if (vec) DGI_LP(float, true); else DGI_LP(float, false); }
+  else { if (vec) DGI_LP(uint16_t, true); else DGI_LP(uint16_t, false); }
+#undef DGI_LP
   DGI_CHECK_LAUNCH();
   return 0;
 }
@@ -299,6 +364,22 @@ extern "C" int dgi_rotate_heads(void* x, int stride, int is_f32, int T, const in
 extern "C" int dgi_gate_heads(void* out, const void* ov, long long ov_hs, long long ov_ts, const void* gate,
                               int gate_stride, int per_head, int T, int H, int dv, int is_f32, hipStream_t s) {
   if (T == 0 || H * dv == 0) return 0;
+  {
+    const int E = is_f32 ? 4 : 8;
+    const bool galign = !gate || per_head || (gate_stride % E == 0 && ((uintptr_t)gate & 15) == 0);
+    if (dv % E == 0 && ov_hs % E == 0 && ov_ts % E == 0 && (((uintptr_t)out | (uintptr_t)ov) & 15) == 0 && galign) {
+      const dim3 vgrid(T, (H * dv / E + NT - 1) / NT);
+      if (vgrid.y > 65535) return -3;
+      if (is_f32)
+        gate_heads_vec_kernel<float><<<vgrid, NT, 0, s>>>((float*)out, (const float*)ov, ov_hs, ov_ts, (const float*)gate,
+                                                         gate_stride, per_head, H, dv);
+      else
+        gate_heads_vec_kernel<uint16_t><<<vgrid, NT, 0, s>>>((uint16_t*)out, (const uint16_t*)ov, ov_hs, ov_ts,
+                                                            (const uint16_t*)gate, gate_stride, per_head, H, dv);
+      DGI_CHECK_LAUNCH();
+      return 0;
+    }
+  }
   const dim3 grid(T, (H * dv + NT - 1) / NT);
   if (grid.y > 65535) return -3;
   if (is_f32)

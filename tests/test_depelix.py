@@ -207,12 +207,13 @@ def test_stream_add_norm(device, dtype, W):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("kr,rd,dims,inter", [(12, 4, 4, False), (8, 6, 4, True), (9, 2, 2, False), (64, 32, 32, True)])
-def test_latent_prep_norms_rotates_and_writes_pages(device, dtype, kr, rd, dims, inter):
+@pytest.mark.parametrize("kr,rd,dims,inter,qr,extra", [(12, 4, 4, False, 10, 3), (8, 6, 4, True, 10, 3), (9, 2, 2, False, 10, 3),
+                                                       (64, 32, 32, True, 10, 3), (64, 32, 32, False, 24, 8), (24, 8, 8, True, 2056, 0)])
+def test_latent_prep_norms_rotates_and_writes_pages(device, dtype, kr, rd, dims, inter, qr, extra):
     """Query latent norm; latent norm + rotary of the key part into scattered page slots; rows with slot -1
     are not written; a layer without a latent of its own computes the query side only."""
     from dgi import ops
-    T, qr, eps, bs, extra = 7, 10, 1e-4, 4, 3
+    T, eps, bs = 7, 1e-4, 4
     proj = rnd(T, qr + kr + rd + extra, seed=5).to(dtype)
     dqw, dkw = rnd(qr, seed=6) + 1, rnd(kr, seed=7) + 1
     pos = torch.tensor([0, 1, 2, 30, 31, 32, 200], dtype=I32)
@@ -344,17 +345,18 @@ def attend_plain_folded(ql, qr, c, r, window, scale, p):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gate_heads_and_gelu(device, dtype):
-    H, T, dv = 3, 5, 7
-    ov = rnd(H, T + 2, dv, seed=20).to(dtype)[:, 1:T + 1]              # a strided [H, T, dv] view
     tol = 1e-6 if dtype == torch.float32 else 0.03
-    for per_head in (True, False):
-        gate = rnd(T, (H if per_head else H * dv) + 3, seed=21).to(dtype)[:, 2:2 + (H if per_head else H * dv)]
-        got = latent.gate_heads(ov.to(device), gate.to(device), per_head)
-        sg = torch.sigmoid(gate.to(F64))
+    for H, T, dv in ((3, 5, 7), (5, 4, 16)):                    # element-wise and 16-byte paths
+        ov = rnd(H, T + 2, dv, seed=20).to(dtype)[:, 1:T + 1]   # a strided [H, T, dv] view
         o = ov.to(F64).permute(1, 0, 2)
-        want = (o * (sg[:, :, None] if per_head else sg.view(T, H, dv))).reshape(T, H * dv)
-        close(got.float(), want, tol)
-    close(latent.gate_heads(ov.to(device), None, True).float(), ov.to(F64).permute(1, 0, 2).reshape(T, H * dv), tol)
+        for per_head in (True, False):
+            n = H if per_head else H * dv
+            gate = rnd(T, n + 8, seed=21).to(dtype)[:, 8 * (dv == 16):][:, :n]      # gate columns inside a wider row
+            got = latent.gate_heads(ov.to(device), gate.to(device), per_head)
+            sg = torch.sigmoid(gate.to(F64))
+            close(got.float(), (o * (sg[:, :, None] if per_head else sg.view(T, H, dv))).reshape(T, H * dv), tol)
+        close(latent.gate_heads(ov.to(device), None, True).float(), o.reshape(T, H * dv), tol)
+    T = 5
     for n in (6, 64):
         x = rnd(T, n, seed=22, scale=2.0).to(dtype)
         close(latent.gelu_tanh(x.to(device)).float(), orc.gelu_tanh(x.to(F64)), tol)
