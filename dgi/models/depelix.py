@@ -29,10 +29,13 @@ Per layer the step executes (rows: decode rows first, then packed prompt portion
     stream_add_norm (HIP)   previous sublayer's residual add (+ the token input's unit-RMS norm) + n1 norm
     D_q | D_kv | gate GEMM  one fused weight
     latent_prep (HIP)       c_q norm; c norm + rotary of the key part -> the paged cache row
-    U_q GEMM, then q_nope -> latent space by a batched GEMM over heads (the key up-projection folded
-                            into the query, so attention runs on the cached rows themselves)
-    latent_attn_rows (HIP)  decode rows and prompt rows, window / causal, rotates the query's rotated part
-    U_v batched GEMM -> gate_heads (HIP: head gate / element gate, heads side by side) -> o GEMM
+    U_q GEMM
+    rows (decode rows, short portions, fp32):  q_nope -> latent space by a batched GEMM over heads (the key
+                            up-projection folded into the query) -> latent_attn_rows (HIP: MFMA for bf16, window /
+                            causal, rotates the query's rotated part) on the cached rows themselves -> U_v batched GEMM
+    long portions (bf16, dim + rot_dim == vdim in {64, 128}):  pages expanded into per-head keys [U_k c | r] and
+                            values U_v c (two GEMMs) -> rotate_heads (HIP) -> MFMA flash kernel with window / causal mask
+    gate_heads (HIP: head gate / element gate, heads side by side) -> o GEMM
     stream_add_norm (HIP)   x += mix, n2 norm
     dense: up GEMM -> gelu_tanh (HIP) -> down GEMM;  moe: router GEMM (fp32) -> moe_route (HIP) -> experts
     stream_add_norm (HIP)   x += ff (-> bf16 copy of x) ; G GEMM -> gelu_tanh x gathered token row (HIP) -> P GEMM

@@ -13,7 +13,9 @@ dims) shared by all heads.  Head h's key is ``[W_uk[h] c | r]`` and its value ``
 
 i.e. with the query folded through W_uk ("q_lat", a batched GEMM over heads before the kernel) the
 attention runs directly on the cached rows, and W_uv is applied once per query to the weighted
-latent sum (a batched GEMM after the kernel).  Nothing per head is ever materialised per key.
+latent sum (a batched GEMM after the kernel).  In this form nothing per head is materialised per key;
+long prompt portions may instead expand their pages into per-head keys and values for the MFMA
+flash kernel (``dgi.models.depelix``), which costs fewer MACs per query and key.
 
 Same rules as ``dgi.ops.mix``: GPU tensors run the HIP kernel (and raise if the library is
 missing), CPU tensors the ``*_ref`` function in fp32, which is also the kernel tests' oracle.
