@@ -245,8 +245,8 @@ __global__ __launch_bounds__(256) void latent_attn_reduce_kernel(const float* __
 // heads and one run of the row's 64-key tiles; its four waves take 16 keys of every tile each and keep
 // their own running softmax, so nothing is exchanged between waves per tile.  Per tile and wave:
 //
-//   S^T [16 keys x 16 heads] = K [16 keys x D] Q^T [D x 16 heads]      D / 16 MFMAs 16x16x16; K rows from LDS,
-//                                                                     Q fragments held in registers
+//   S^T [16 keys x 16 heads] = K [16 keys x D] Q^T [D x 16 heads]      D / 16 MFMAs 16x16x16; K rows from LDS;
+//                                                                     Q rows stay in LDS beside the tile
 //   O^T [kr x 16 heads]     += C^T [kr x 16 keys] P^T [16 keys x 16 heads]    kr / 16 MFMAs
 //
 // S^T comes out with a lane holding four consecutive keys of one head, which is exactly the operand
@@ -263,7 +263,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     uint16_t* __restrict__ out, long long o_hs, long long o_ts, float* __restrict__ part_o, float* __restrict__ part_ml,
     unsigned cpr_magic) {
   constexpr int KT = 64;
-  extern __shared__ __attribute__((aligned(16))) uint16_t tile[];       // [KT][DP]; first holds the 16 queries
+  extern __shared__ __attribute__((aligned(16))) uint16_t qs[];         // [16][DP] the group's queries, then the tile
+  uint16_t* tile = qs + (size_t)16 * DP;                                 // [KT][DP]
   const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int lr = lane & 15, lg = lane >> 4;
   const int D = kr + rd, nd = D >> 4, nm = kr >> 4;
@@ -299,14 +300,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
           const int head = g * 16 + hh;
           u32x4 v = {0u, 0u, 0u, 0u};
           if (head < H) v = *reinterpret_cast<const u32x4*>(q_lat + (size_t)head * ql_hs + (size_t)row * ql_ts + c * 8);
-          *reinterpret_cast<u32x4*>(tile + (size_t)hh * DP + c * 8) = v;
+          *reinterpret_cast<u32x4*>(qs + (size_t)hh * DP + c * 8) = v;
         }
       }
     } else {
       for (int i = threadIdx.x; i < 16 * kr; i += 256) {
         const int hh = i / kr, e = i - hh * kr;
         const int head = g * 16 + hh;
-        tile[(size_t)hh * DP + e] = head < H ? q_lat[(size_t)head * ql_hs + (size_t)row * ql_ts + e] : (uint16_t)0;
+        qs[(size_t)hh * DP + e] = head < H ? q_lat[(size_t)head * ql_hs + (size_t)row * ql_ts + e] : (uint16_t)0;
       }
     }
     // rotated part
@@ -329,16 +330,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
           v = qr[e2];
         }
       }
-      tile[(size_t)hh * DP + kr + e2] = v;
+      qs[(size_t)hh * DP + kr + e2] = v;
     }
   }
   __syncthreads();
-  short4v qf[NDS];
-#pragma unroll
-  for (int s = 0; s < NDS; ++s) {
-    qf[s] = short4v{0, 0, 0, 0};
-    if (s < nd) qf[s] = *reinterpret_cast<const short4v*>(tile + (size_t)lr * DP + 16 * s + 4 * lg);
-  }
+  const uint16_t* qp = qs + (size_t)lr * DP + 4 * lg;   // this lane's operand of Q^T: head lr, dims 16 s + 4 lg .. + 3
 
   float m_run = -__builtin_inff(), l_run = 0.f;        // of head lr, over this wave's keys
   f32x4 acc[NM];                                       // O^T: latent dims 16 m + 4 lg + i of head lr
@@ -372,7 +368,6 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     }
   };
   const int t_lo = blockIdx.z * tps;
-  __syncthreads();                                     // every wave has its query fragments: the tile region is free
   if (t_lo < t_hi) issue(t_lo);
   for (int ti = t_lo; ti < t_hi; ++ti) {
     const int k0 = first + ti * KT;
@@ -396,7 +391,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     for (int s = 0; s < NDS; ++s) {
       if (s < nd) {
         const short4v a = *reinterpret_cast<const short4v*>(kp + 16 * s);
-        sp[s & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sp[s & 3], 0, 0, 0);
+        const short4v b = *reinterpret_cast<const short4v*>(qp + 16 * s);
+        sp[s & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, sp[s & 3], 0, 0, 0);
       }
     }
     f32x4 sc;
@@ -561,7 +557,7 @@ int launch_mfma(const void* q, int q_stride, const void* q_lat, long long ql_hs,
   const unsigned magic = (unsigned)((0x100000000ull + cpr - 1) / cpr);
   for (unsigned i = 0; i < 16 * cpr + 64; ++i)
     if ((unsigned)(((unsigned long long)i * magic) >> 32) != i / cpr) return -9;
-  const size_t lds = std::max((size_t)64 * DP * 2, (size_t)(160 + 16 * (kr + 4)) * 4);     // tiles, then the combine buffers
+  const size_t lds = (size_t)16 * DP * 2 + std::max((size_t)64 * DP * 2, (size_t)(160 + 16 * (kr + 4)) * 4);     // queries; tiles, then the combine buffers
   if (lds > lds_max()) return -6;
   static int allowed = -1;
   if (allowed != 0 && lds > 64 * 1024) {
