@@ -350,14 +350,18 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
   // computed: the loads' latency hides behind the MFMAs.
   constexpr int NLD = (16 * NDS * 2 + 63) / 64;        // 16-byte chunks per lane: 16 rows of at most NDS * 2 chunks
   u32x4 pre[NLD];
+  // lane j < 16 resolves the cache slot of the wave's row j of a tile (-1: past the last key); the slots of
+  // tile t + 1 are looked up while tile t's rows are fetched, so the page-table read is off the critical path
+  auto slot_of = [&](int ti) {
+    const int key = first + ti * KT + 16 * w + lane;
+    int sl = -1;
+    if (lane < 16 && ti < t_hi && key <= pos) sl = bt[key / bs] * bs + (key % bs);
+    return sl;
+  };
+  int next_slot = slot_of(blockIdx.z * tps);
   auto issue = [&](int ti) {
-    const int k0 = first + ti * KT + 16 * w;
-    // lane j < 16 resolves the cache slot of the wave's row j once; the chunk loads fetch it by shuffle
-    int myslot = -1;                                   // rows past the last key: none
-    if (lane < 16 && k0 + lane <= pos) {
-      const int key = k0 + lane;
-      myslot = bt[key / bs] * bs + (key % bs);
-    }
+    const int myslot = next_slot;
+    next_slot = slot_of(ti + 1);
 #pragma unroll
     for (int it = 0; it < NLD; ++it) {
       const int idx = lane + 64 * it;
@@ -439,11 +443,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     }
     __builtin_amdgcn_wave_barrier();                   // this tile's rows are read before the next ones land
   }
-  // combine the four waves: every head's (max, sum) through LDS, then O^T summed wave after wave in LDS
+  // combine the four waves: every head's (max, sum) through LDS; O^T of waves 0 / 1 into two LDS buffers, waves
+  // 2 / 3 added on top, and the output pass adds the two buffers
   __syncthreads();                                     // the last tile is fully read
   float* ml = reinterpret_cast<float*>(tile);          // [4 waves][16 heads][2], then [16 heads][2] combined
-  float* os = ml + 160;                                // [16 heads][kr + 4] fp32
   const int ks = kr + 4;                               // padded: a head's rows start 4 banks apart
+  float* os = ml + 160;                                // [2][16 heads][ks] fp32
   if (lg == 0) {
     ml[(w * 16 + lr) * 2] = m_run;
     ml[(w * 16 + lr) * 2 + 1] = l_run;
@@ -459,13 +464,15 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     Lsum += mw == -__builtin_inff() ? 0.f : ml[(ww * 16 + lr) * 2 + 1] * expf(mw - M);
   }
   const float f = m_run == -__builtin_inff() ? 0.f : expf(m_run - M);     // a wave (or a whole run) without keys adds nothing
-  for (int ww = 0; ww < 4; ++ww) {
-    if (w == ww) {
+  float* mine = os + (w & 1) * 16 * ks + lr * ks + 4 * lg;
+#pragma unroll
+  for (int ph = 0; ph < 2; ++ph) {
+    if ((w >> 1) == ph) {
 #pragma unroll
       for (int m = 0; m < NM; ++m) {
         if (m < nm) {
-          float4* dst = reinterpret_cast<float4*>(os + (size_t)lr * ks + 16 * m + 4 * lg);
-          float4 cur = ww == 0 ? make_float4(0.f, 0.f, 0.f, 0.f) : *dst;
+          float4* dst = reinterpret_cast<float4*>(mine + 16 * m);
+          float4 cur = ph == 0 ? make_float4(0.f, 0.f, 0.f, 0.f) : *dst;
           cur.x += acc[m][0] * f; cur.y += acc[m][1] * f; cur.z += acc[m][2] * f; cur.w += acc[m][3] * f;
           *dst = cur;
         }
@@ -473,25 +480,36 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     }
     __syncthreads();
   }
-  if (w == 0 && lg == 0) {                             // every wave has read the per-wave entries before the barriers above
-    ml[128 + lr * 2] = M;
-    ml[128 + lr * 2 + 1] = Lsum;
-  }
-  __syncthreads();
-  for (int i = threadIdx.x; i < 16 * kr; i += 256) {
-    const int hh = i / kr, e = i - hh * kr;
-    const int head = g * 16 + hh;
-    if (head >= H) break;
-    const float v = os[(size_t)hh * ks + e];
-    if (part_o) {
-      const size_t slot = ((size_t)blockIdx.z * H + head) * rows + row;
-      part_o[slot * kr + e] = v;
-      if (e == 0) {
-        part_ml[2 * slot] = ml[128 + hh * 2];
-        part_ml[2 * slot + 1] = ml[128 + hh * 2 + 1];
+  // 16 threads per head, four consecutive latent dims each
+  const int hh = threadIdx.x >> 4, part = threadIdx.x & 15;
+  const int head = g * 16 + hh;
+  if (head >= H) return;
+  // (M, Lsum) of head hh live in the lanes with lr == hh: lane hh of this thread's wave has them
+  const float Mh = __shfl(M, hh, 64), Lh = __shfl(Lsum, hh, 64);
+  const float* o0 = os + hh * ks;
+  const float* o1 = o0 + 16 * ks;
+  if (part_o) {
+    const size_t slot = ((size_t)blockIdx.z * H + head) * rows + row;
+    for (int e = part * 4; e < kr; e += 64) {
+      const float4 x = *reinterpret_cast<const float4*>(o0 + e), y = *reinterpret_cast<const float4*>(o1 + e);
+      *reinterpret_cast<float4*>(part_o + slot * kr + e) = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+    }
+    if (part == 0) {
+      part_ml[2 * slot] = Mh;
+      part_ml[2 * slot + 1] = Lh;
+    }
+  } else {
+    const float inv = 1.f / Lh;
+    uint16_t* op = out + (size_t)head * o_hs + (size_t)row * o_ts;
+    const bool ovec = ((uintptr_t)out & 7) == 0 && (o_hs & 3) == 0 && (o_ts & 3) == 0;
+    for (int e = part * 4; e < kr; e += 64) {
+      const float4 x = *reinterpret_cast<const float4*>(o0 + e), y = *reinterpret_cast<const float4*>(o1 + e);
+      const float v0 = (x.x + y.x) * inv, v1 = (x.y + y.y) * inv, v2 = (x.z + y.z) * inv, v3 = (x.w + y.w) * inv;
+      if (ovec) {
+        *reinterpret_cast<uint2*>(op + e) = make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+      } else {
+        op[e] = f32_to_bf16(v0); op[e + 1] = f32_to_bf16(v1); op[e + 2] = f32_to_bf16(v2); op[e + 3] = f32_to_bf16(v3);
       }
-    } else {
-      out[(size_t)head * o_hs + (size_t)row * o_ts + e] = f32_to_bf16(v / ml[128 + hh * 2 + 1]);
     }
   }
 }
@@ -557,7 +575,7 @@ int launch_mfma(const void* q, int q_stride, const void* q_lat, long long ql_hs,
   const unsigned magic = (unsigned)((0x100000000ull + cpr - 1) / cpr);
   for (unsigned i = 0; i < 16 * cpr + 64; ++i)
     if ((unsigned)(((unsigned long long)i * magic) >> 32) != i / cpr) return -9;
-  const size_t lds = (size_t)16 * DP * 2 + std::max((size_t)64 * DP * 2, (size_t)(160 + 16 * (kr + 4)) * 4);     // queries; tiles, then the combine buffers
+  const size_t lds = (size_t)16 * DP * 2 + std::max((size_t)64 * DP * 2, (size_t)(160 + 32 * (kr + 4)) * 4);     // queries; tiles, then the combine buffers
   if (lds > lds_max()) return -6;
   static int allowed = -1;
   if (allowed != 0 && lds > 64 * 1024) {
