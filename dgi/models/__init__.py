@@ -1,4 +1,5 @@
-from dgi.models.config import (BebovikConfig, DepelixConfig, ModelConfig, PRESETS, TifepelConfig,  # noqa: F401
+from dgi.models.config import (BebovikConfig, DepelixConfig, LofuvikConfig, ModelConfig, PRESETS,  # noqa: F401
+                               TifepelConfig,
                                get_config)
 
 
@@ -13,6 +14,9 @@ def model_class(cfg):
     if isinstance(cfg, DepelixConfig):
         from dgi.models.depelix import DepelixModel
         return DepelixModel
+    if isinstance(cfg, LofuvikConfig):
+        from dgi.models.lofuvik import LofuvikModel
+        return LofuvikModel
     from dgi.models.llama import LlamaModel
     return LlamaModel
 

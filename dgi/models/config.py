@@ -125,8 +125,9 @@ class ModelConfig:
 class RotarySpec:
     """Rotary position parameters of one attention mixer: the first ``dims`` dimensions of a
     head rotate in pairs at frequency base^(-2i/dims) — ``layout`` "interleaved" pairs (2i, 2i+1),
-    "half" pairs (i, i + dims/2); ``scaling`` (factor, low, high, original) rescales the
-    frequencies by wavelength, or None."""
+    "half" pairs (i, i + dims/2); ``scaling`` rescales the frequencies by wavelength, or None:
+    (factor, low, high, original) the stepwise form, (factor, original, fast, slow) the ramp form
+    that also stretches cos and sin (``dgi.ops.rope_cos_sin``)."""
     base: float
     dims: int
     scaling: Optional[dict] = None
@@ -155,6 +156,11 @@ class AttentionSpec:
     # ``distance_bucket(i - j, bias_rows, bias_max)`` (bias_rows 0: none)
     bias_rows: int = 0
     bias_max: float = 0.0
+    # "head": q and k are RMS-normed per head with a weight of ``dim`` entries; "full": over the whole
+    # projection (all heads at once) with a weight as long as the projection
+    qk_norm: str = "head"
+    softcap: float = 0.0         # scaled scores s become softcap * tanh(s / softcap) (0: none)
+    sink: bool = False           # a learned per-head logit joins the softmax denominator (no key, no value)
 
     @property
     def q_size(self) -> int:
@@ -223,7 +229,9 @@ class MoeSpec:
     ``identity`` experts that return their input; a token takes the ``top`` experts with the
     largest softmax score + selection bias and weighs them by the plain scores (not
     renormalised).  ``shared_ff`` > 0: a shared expert of that width runs for every token.
-    ``score`` "sigmoid": independent sigmoid scores instead of the softmax.  ``act`` "clamped":
+    ``score`` "sigmoid": independent sigmoid scores instead of the softmax; "top_softmax": the
+    ``top`` largest logits are taken and their weights are the softmax over those alone.
+    ``router_bias``: the router has a bias that is part of the logits.  ``act`` "clamped":
     experts are clamped sigmoid-GLUs (``GluSpec`` with ``limit``) instead of gated SiLU.
     ``weigh`` "input": the route weight multiplies the expert's input, not its output."""
     experts: int
@@ -237,6 +245,7 @@ class MoeSpec:
     limit: float = 0.0
     weigh: str = "output"
     selection_bias: bool = True     # a learned per-route bias is added to the scores for the choice only
+    router_bias: bool = False
 
     @property
     def routes(self) -> int:
@@ -301,9 +310,77 @@ class DenseSpec:
 
 
 @dataclasses.dataclass
+class WkvSpec:
+    """One RWKV-style time-mixing layer: ``heads`` heads whose receptance, key and value all have
+    ``dim`` channels; every projection reads its own blend of the current and the previous input
+    (static per-channel coefficients); the per-channel decay comes from a low-rank projection of
+    ``decay_rank`` dims (0: read from the checkpoint's tensor shape); the current token gets a
+    per-channel bonus instead of the decayed state."""
+    heads: int
+    dim: int
+    decay_rank: int = 0
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.dim
+
+
+@dataclasses.dataclass
+class DeltaSpec:
+    """One gated delta-rule layer: ``kv_heads`` query/key heads of ``dim`` channels shared by
+    ``heads`` value heads of ``vdim``; q, k and v pass a causal convolution of ``conv`` taps and
+    SiLU; per head one decay and one write strength per token."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+
+    @property
+    def qk_size(self) -> int:
+        return self.kv_heads * self.dim
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.qk_size + self.inner
+
+
+@dataclasses.dataclass
+class MlstmSpec:
+    """One matrix-memory (mLSTM) layer: ``heads`` heads with ``dim`` query/key and ``vdim`` value
+    channels, exponential input gate and sigmoid forget gate in log space, both soft-capped at
+    ``gate_cap``, with a running maximum as stabiliser and a normaliser vector."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+    @property
+    def qk_size(self) -> int:
+        return self.heads * self.dim
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+
+@dataclasses.dataclass
+class ParallelSpec:
+    """Two mixers side by side on the same input: ``left`` softmax attention (``AttentionSpec``),
+    ``right`` a matrix memory (``MlstmSpec``); the result is the mean of the two outputs, each
+    RMS-normed over the model width with its own weight."""
+    left: AttentionSpec
+    right: MlstmSpec
+
+
+@dataclasses.dataclass
 class LayerSpec:
     type: str
-    mixer: object                     # AttentionSpec | Mamba2Spec | LatentAttentionSpec
+    mixer: object                     # AttentionSpec | Mamba2Spec | LatentAttentionSpec | WkvSpec | DeltaSpec | ParallelSpec
     mlp: Optional[object] = None      # GluSpec | MoeSpec | DenseSpec
 
 
@@ -717,8 +794,175 @@ def depelix_uniform(name: str, vocab: int, width: int, pattern: str, heads: int,
     return DepelixConfig(name=name, vocab_size=vocab, hidden_size=width, layers=layers, side_dim=side_dim, **kw)
 
 
+@dataclasses.dataclass
+class LofuvikConfig:
+    """A Lofuvik decoder: plain token embedding, one fp32 stream, layers of the parallel form
+    ``x += Mix(h) + FF(h)`` with ``h = RMSnorm(x)``, where Mix is RWKV-style time mixing
+    (``WkvSpec``), a gated delta rule (``DeltaSpec``) or softmax attention with a sink beside a
+    matrix memory (``ParallelSpec``), and FF a mixture of experts chosen by the largest router
+    logits (or none).  A span of layers (``loop_start`` .. ``loop_stop`` - 1) runs ``loop_times``
+    times with the same weights; every pass has its own cache and state, and every pass but the
+    first starts by adding the embedding output to the stream."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: list
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    norm_eps: float = 1e-6
+    max_position: int = 2048
+    bos_token_id: int = -1
+    eos_token_id: int = -1
+    arch: str = "lofuvik"
+    tie_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def layer_runs(self) -> list:
+        """Layer index of every layer run, in execution order."""
+        n = len(self.layers)
+        if self.loop_times <= 1 or self.loop_stop <= self.loop_start:
+            return list(range(n))
+        a, b = self.loop_start, self.loop_stop
+        return list(range(a)) + list(range(a, b)) * self.loop_times + list(range(b, n))
+
+    @property
+    def pass_starts(self) -> set:
+        """Run indices at which a repeated pass begins (the embedding output is added there)."""
+        if self.loop_times <= 1 or self.loop_stop <= self.loop_start:
+            return set()
+        a, b = self.loop_start, self.loop_stop
+        return {a + k * (b - a) for k in range(1, self.loop_times)}
+
+    def _attn(self):
+        return [l.mixer.left for l in self.layers if l.type == "parallel"]
+
+    @property
+    def num_heads(self) -> int:
+        return max([m.heads for m in self._attn()] or [1])
+
+    @property
+    def num_kv_heads(self) -> int:
+        return max([m.kv_heads for m in self._attn()] or [1])
+
+    @property
+    def head_dim(self) -> int:
+        return max([max(m.dim, m.vdim) for m in self._attn()] or [1])
+
+    @property
+    def rms_eps(self) -> float:
+        return self.norm_eps
+
+    def kv_layer_shapes(self, start: int = 0, end: Optional[int] = None) -> list:
+        """(kv heads, key size, value size) of the cache pages of every attention RUN (a looped
+        layer has pages per pass); the recurrent mixers hold no pages."""
+        return [(self.layers[li].mixer.left.kv_heads, self.layers[li].mixer.left.dim, self.layers[li].mixer.left.vdim)
+                for li in self.layer_runs if self.layers[li].type == "parallel"]
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2, layers: Optional[int] = None) -> int:
+        return sum(g * (dk + dv) for g, dk, dv in self.kv_layer_shapes()) * dtype_bytes
+
+    def param_count(self) -> int:
+        W = self.hidden_size
+        n = 2 * self.vocab_size * W
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "wkv":
+                n += 5 * W * m.inner + 2 * m.decay_rank * (W + m.inner) // 2
+            elif l.type == "delta":
+                n += W * (2 * m.qk_size + 3 * m.inner + 2 * m.heads)
+            else:
+                a, r = m.left, m.right
+                n += W * (a.q_size + a.k_size + a.v_size + 2 * a.o_size) + W * (2 * r.qk_size + 3 * r.inner + 2 * r.heads)
+            f = l.mlp
+            if f is not None:
+                n += 3 * W * f.ff * f.experts + W * f.routes
+        return n
+
+    def to_dict(self) -> dict:
+        return dataclasses.asdict(self)
+
+    @staticmethod
+    def from_dict(d: dict, name: str = "lofuvik") -> "LofuvikConfig":
+        layers = []
+        for e in d["layers"]:
+            m, kind = e["mixer"], e["type"]
+            if kind == "wkv":
+                spec = WkvSpec(heads=int(m["heads"]), dim=int(m["dim"]), decay_rank=int(m.get("decay_rank") or 0))
+            elif kind == "delta":
+                spec = DeltaSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                 vdim=int(m["vdim"]), conv=int(m["conv"]))
+                if spec.heads % spec.kv_heads:
+                    raise ValueError("Lofuvik: heads must be a multiple of kv_heads")
+            elif kind == "parallel":
+                a, r = m["left"], m["right"]
+                rot = a.get("rot")
+                left = AttentionSpec(
+                    heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                    scale=float(a["scale"]),
+                    rot=None if not rot or not int(rot.get("dims") or 0) else
+                    RotarySpec(float(rot["base"]), int(rot["dims"]), rot.get("scaling") or None, "half"),
+                    out_gate=True, qk_norm="full", softcap=float(a.get("softcap") or 0.0), sink=True)
+                if left.heads % left.kv_heads:
+                    raise ValueError("Lofuvik: heads must be a multiple of kv_heads")
+                if left.rot is not None and (left.rot.dims > left.dim or left.rot.dims % 2):
+                    raise ValueError("Lofuvik: rot.dims must be even and at most dim")
+                spec = ParallelSpec(left, MlstmSpec(heads=int(r["heads"]), dim=int(r["dim"]), vdim=int(r["vdim"]),
+                                                    gate_cap=float(r["gate_cap"])))
+            else:
+                raise ValueError(f"Lofuvik: unknown mixer type {kind!r}")
+            f = e.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind", "moe") != "moe":
+                    raise ValueError(f"Lofuvik: unknown feed-forward kind {f.get('kind')!r}")
+                r = f["router"]
+                mlp = MoeSpec(experts=int(r["experts"]), identity=0, top=int(r["top"]), ff=int(f["expert"]["ff"]),
+                              score="top_softmax", selection_bias=False, router_bias=True)
+                if not 1 <= mlp.top <= mlp.experts:
+                    raise ValueError("Lofuvik: router.top must be between 1 and router.experts")
+            layers.append(LayerSpec(kind, spec, mlp))
+        lp = d.get("loop") or {}
+        return LofuvikConfig(
+            name=name, vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), layers=layers,
+            loop_start=int(lp.get("start") or 0), loop_stop=int(lp.get("stop") or 0), loop_times=int(lp.get("times") or 1),
+            norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)), max_position=int(d.get("max_positions") or 2048))
+
+
+def lofuvik_uniform(name: str, vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, vdim: int,
+                    r_heads: int, r_dim: int, r_vdim: int, experts: int, top: int, ff: int, conv: int = 4,
+                    decay_rank: int = 32, rot_dims: Optional[int] = None, base: float = 10000.0,
+                    scaling: Optional[dict] = None, softcap: float = 30.0, gate_cap: float = 15.0, **kw) -> LofuvikConfig:
+    """A Lofuvik configuration from a layer pattern: 'd' gated delta rule, 'p' attention beside a
+    matrix memory, 'w' RWKV-style time mixing; upper case: the layer has no feed-forward.
+    ``heads`` / ``kv_heads`` / ``dim`` / ``vdim`` size the attention, ``r_*`` the recurrent mixers
+    (the delta rule's q/k heads are ``r_heads // 2``, at least one); presets and benchmarks."""
+    layers = []
+    for ch in pattern:
+        k = ch.lower()
+        if k == "w":
+            mixer, kind = WkvSpec(r_heads, r_dim, decay_rank), "wkv"
+        elif k == "d":
+            mixer, kind = DeltaSpec(r_heads, max(1, r_heads // 2), r_dim, r_vdim, conv), "delta"
+        elif k == "p":
+            rd = dim if rot_dims is None else rot_dims
+            left = AttentionSpec(heads, kv_heads, dim, vdim, dim ** -0.5,
+                                 RotarySpec(base, rd, scaling, "half") if rd else None, out_gate=True, qk_norm="full",
+                                 softcap=softcap, sink=True)
+            mixer, kind = ParallelSpec(left, MlstmSpec(r_heads, r_dim, r_vdim, gate_cap)), "parallel"
+        else:
+            raise ValueError(f"lofuvik_uniform: unknown layer kind {ch!r}")
+        layers.append(LayerSpec(kind, mixer, MoeSpec(experts, 0, top, ff, score="top_softmax", selection_bias=False,
+                                                     router_bias=True) if ff and ch.islower() else None))
+    return LofuvikConfig(name=name, vocab_size=vocab, hidden_size=width, layers=layers, **kw)
+
+
 NATIVE_CONFIGS = {"bebovik": BebovikConfig.from_dict, "tifepel": TifepelConfig.from_dict,
-                  "depelix": DepelixConfig.from_dict}
+                  "depelix": DepelixConfig.from_dict, "lofuvik": LofuvikConfig.from_dict}
 
 
 PRESETS: dict[str, ModelConfig] = {
@@ -774,6 +1018,13 @@ PRESETS: dict[str, ModelConfig] = {
     "depelix-tiny": depelix_uniform("depelix-tiny", 512, 128, "wScW", 4, 16, 16, 24, 48, 64, 40, 256, experts=6, top=2,
                                     expert_ff=64, limit=2.0, side_dim=16, bigram_buckets=251, bigram_mul_prev=31,
                                     bigram_mul_cur=7, max_position=2048, bos_token_id=1, eos_token_id=2),
+    # Lofuvik test / smoke sizes (random weights): delta rule, attention + matrix memory, time mixing; the
+    # first two layers run twice
+    "lofuvik-tiny": lofuvik_uniform("lofuvik-tiny", 512, 128, "dpwD", 4, 2, 32, 48, 4, 16, 32, 6, 2, 64, conv=3,
+                                    decay_rank=8, rot_dims=16, base=10000.0,
+                                    scaling={"factor": 2.0, "original": 64, "fast": 8.0, "slow": 1.0},
+                                    loop_start=0, loop_stop=2, loop_times=2, max_position=2048,
+                                    bos_token_id=1, eos_token_id=2),
     "opt-125m": ModelConfig(name="opt-125m", arch="opt", vocab_size=50272, hidden_size=768,
                             intermediate_size=3072, num_layers=12, num_heads=12, num_kv_heads=12, head_dim=64,
                             max_position=2048, tie_embeddings=True, bos_token_id=2, eos_token_id=2),
@@ -803,7 +1054,7 @@ def get_config(name_or_path: str) -> ModelConfig:
     if "@L" in name_or_path:
         base, n = name_or_path.rsplit("@L", 1)
         bc = get_config(base)
-        if isinstance(bc, (BebovikConfig, TifepelConfig, DepelixConfig)):
+        if isinstance(bc, (BebovikConfig, TifepelConfig, DepelixConfig, LofuvikConfig)):
             return dataclasses.replace(bc, name=name_or_path, layers=bc.layers[: int(n)])
         return dataclasses.replace(bc, name=name_or_path, num_layers=int(n))
     key = ALIASES.get(name_or_path, name_or_path)

@@ -359,3 +359,94 @@ def load_depelix_checkpoint(model, path: str) -> dict:
     out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
     rd.close()
     return out
+
+
+def lofuvik_checkpoint_shapes(cfg, path: str) -> None:
+    """Sizes that only the checkpoint's tensor shapes give: the rank of every time-mixing layer's
+    decay projection (rows of ``l<i>.mix.w1``)."""
+    rd = CheckpointReader(path)
+    for i, l in enumerate(cfg.layers):
+        if l.type == "wkv":
+            name = f"l{i}.mix.w1"
+            l.mixer.decay_rank = int(rd._h(name).get_slice(name).get_shape()[0])
+    rd.close()
+
+
+def load_lofuvik_checkpoint(model, path: str) -> dict:
+    """Fill a ``LofuvikModel`` from the design's safetensors layout: ``embed`` / ``head`` / ``final.norm`` and
+    per layer i ``l<i>.norm1``, the feed-forward under ``l<i>.mlp.`` (router, router.b, e<j>.{gate,up,down})
+    and the mixer under ``l<i>.mix.``: time mixing mu.{r,k,v,g,w}, r, k, v, g, w1, w2, w0, u, norm, o; delta
+    rule q, k, v (each with ``.conv``), b, a, A_log, dt_bias, norm, g, o; the two-branch mixer left.{q, k, v,
+    q.norm, k.norm, sink, g, o, out} and right.{q, k, v, g, o, norm, i, i.b, f, f.b, out}.  The router and
+    the recurrence's gate projections land in one fp32 side projection (router | b | a, or router | i | f),
+    a mixer's large projections in one fused weight, every expert's gate | up in one stacked tensor; norm
+    weights, blends, taps, decay and gate parameters stay fp32."""
+    rd = CheckpointReader(path)
+    n = 0
+
+    def put(dst, name):
+        nonlocal n
+        src = rd.read(name)
+        if tuple(src.shape) != tuple(dst.shape) and src.numel() != dst.numel():
+            raise ValueError(f"{name}: checkpoint shape {tuple(src.shape)} does not fit {tuple(dst.shape)}")
+        _put(dst, src.reshape(dst.shape))
+        n += 1
+
+    def put_rows(dst, names):
+        r = 0
+        for name, rows in names:
+            put(dst[r:r + rows], name)
+            r += rows
+        if r != dst.shape[0]:
+            raise ValueError(f"{names[0][0]}...: {r} rows for a slot of {dst.shape[0]}")
+
+    from dgi.models.lofuvik import SHIFT_BLENDS
+    for i, L in enumerate(model.layers):
+        p = f"l{i}."
+        x = p + "mix."
+        m, f = L.spec.mixer, L.spec.mlp
+        put(L.norm1, p + "norm1")
+        r0 = 0
+        if f is not None:
+            put(L.side[: f.routes], p + "mlp.router")
+            put(L.side_b[: f.routes], p + "mlp.router.b")
+            r0 = f.routes
+            for e in range(f.experts):
+                put(L.gate_up[e, : f.ff], f"{p}mlp.e{e}.gate")
+                put(L.gate_up[e, f.ff:], f"{p}mlp.e{e}.up")
+                put(L.down[e], f"{p}mlp.e{e}.down")
+        if L.spec.type == "wkv":
+            for j, s in enumerate(SHIFT_BLENDS):
+                put(L.mu[j], x + "mu." + s)
+            for j, s in enumerate(("r", "k", "v", "g")):
+                put(L.rkvg[j], x + s)
+            for dst, key in ((L.w1, "w1"), (L.w2, "w2"), (L.w0, "w0"), (L.bonus, "u"), (L.mnorm, "norm"), (L.o, "o")):
+                put(dst, x + key)
+        elif L.spec.type == "delta":
+            H, qk = m.heads, m.qk_size
+            put_rows(L.in_proj, [(x + "q", qk), (x + "k", qk), (x + "v", m.inner), (x + "g", m.inner)])
+            put_rows(L.conv, [(x + "q.conv", qk), (x + "k.conv", qk), (x + "v.conv", m.inner)])
+            put(L.side[r0: r0 + H], x + "b")
+            put(L.side[r0 + H: r0 + 2 * H], x + "a")
+            for dst, key in ((L.a_log, "A_log"), (L.dt_bias, "dt_bias"), (L.mnorm, "norm"), (L.o, "o")):
+                put(dst, x + key)
+        else:
+            a, rr = m.left, m.right
+            lf, rt = x + "left.", x + "right."
+            put_rows(L.in_proj, [(lf + "q", a.q_size), (lf + "k", a.k_size), (lf + "v", a.v_size), (lf + "g", a.o_size),
+                                 (rt + "q", rr.qk_size), (rt + "k", rr.qk_size), (rt + "v", rr.inner), (rt + "g", rr.inner)])
+            H = rr.heads
+            put(L.side[r0: r0 + H], rt + "i")
+            put(L.side[r0 + H: r0 + 2 * H], rt + "f")
+            put(L.side_b[r0: r0 + H], rt + "i.b")
+            put(L.side_b[r0 + H: r0 + 2 * H], rt + "f.b")
+            for dst, name in ((L.q_norm, lf + "q.norm"), (L.k_norm, lf + "k.norm"), (L.sink, lf + "sink"), (L.o, lf + "o"),
+                              (L.out_left, lf + "out"), (L.o_right, rt + "o"), (L.rnorm, rt + "norm"),
+                              (L.out_right, rt + "out")):
+                put(dst, name)
+    put(model.embed, "embed")
+    put(model.head, "head")
+    put(model.final_norm, "final.norm")
+    out = {"tensors": n, "bytes": rd.bytes_read, "path": path}
+    rd.close()
+    return out

@@ -119,9 +119,28 @@ def rope_cos_sin(head_dim: int, max_pos: int, theta: float, scaling: Optional[di
                  device=None) -> torch.Tensor:
     """[max_pos, head_dim] fp32 table: first half cos, second half sin.
 
-    Supports Llama-3.1 style ``rope_scaling`` (``rope_type == "llama3"``).
+    Supports Llama-3.1 style ``rope_scaling`` (``rope_type == "llama3"``) and the ramp form
+    (keys factor, original, fast, slow): with d(t) = head_dim * ln(original / (2 pi t)) / (2 ln theta),
+    lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), head_dim - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * ramp_i +
+    f_i * (1 - ramp_i), and cos and sin are both multiplied by 0.1 * ln(factor) + 1.
     """
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))
+    if scaling and "fast" in scaling and "slow" in scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def turn_dim(turns: float) -> float:
+            return head_dim * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(theta))
+
+        lo = max(math.floor(turn_dim(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(turn_dim(float(scaling["slow"]))), head_dim - 1)
+        i = torch.arange(head_dim // 2, dtype=torch.float64)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        inv = inv / factor * ramp + inv * (1.0 - ramp)
+        t = torch.arange(max_pos, dtype=torch.float64)
+        f = torch.outer(t, inv)
+        stretch = 0.1 * math.log(factor) + 1.0
+        return (torch.cat([f.cos(), f.sin()], dim=-1) * stretch).float().to(device)
     if scaling and (scaling.get("rope_type", scaling.get("type")) == "llama3" or "original" in scaling):
         # wavelength-dependent rescale; HF key names, or the short ones (factor, low, high, original)
         factor = scaling["factor"]

@@ -39,11 +39,13 @@ def _unit_rms(v: torch.Tensor, eps: float) -> torch.Tensor:
     return v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
 
 
-def stream_add_norm_ref(x, y, post_w, next_w, eps, out_dtype):
+def stream_add_norm_ref(x, y, post_w, next_w, eps, out_dtype, y2=None):
     if y is not None:
         v = y.float()
         if post_w is not None:
             v = _unit_rms(v, eps) * post_w
+        if y2 is not None:
+            v = v + y2.float()
         x.add_(v)
     if out_dtype is None:
         return None
@@ -51,15 +53,18 @@ def stream_add_norm_ref(x, y, post_w, next_w, eps, out_dtype):
 
 
 def stream_add_norm(x: torch.Tensor, y: Optional[torch.Tensor], post_w: Optional[torch.Tensor],
-                    next_w: Optional[torch.Tensor], eps: float, out_dtype=None) -> Optional[torch.Tensor]:
+                    next_w: Optional[torch.Tensor], eps: float, out_dtype=None,
+                    y2: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """One pass over the fp32 stream ``x`` [T, W] (updated in place): ``x += y`` — with ``post_w``:
     ``x += y / rms(y) * post_w`` — then, if ``out_dtype`` is given, returns ``x / rms(x) * next_w``
-    (``next_w`` None: x itself) in that dtype, the next GEMM's input.  rms(v) = sqrt(mean(v^2) + eps)."""
+    (``next_w`` None: x itself) in that dtype, the next GEMM's input.  rms(v) = sqrt(mean(v^2) + eps).
+    ``y2`` (needs ``y``): a second addend of the same step, ``x += y + y2`` (two sublayers that read
+    the same input)."""
     if _native(x):
         out = torch.empty(x.shape, dtype=out_dtype, device=x.device) if out_dtype is not None else None
-        _call("stream_add_norm", x, y, post_w, next_w, float(eps), out)
+        _call("stream_add_norm", x, y, post_w, next_w, float(eps), out, y2)
         return out
-    return stream_add_norm_ref(x, y, post_w, next_w, eps, out_dtype)
+    return stream_add_norm_ref(x, y, post_w, next_w, eps, out_dtype, y2)
 
 
 # ----------------------------------------------------------------------------

@@ -125,23 +125,40 @@ def _rot_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
     return torch.cat([r, x[..., rd:]], dim=-1)
 
 
+def _rot_halves(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """Half-split rotation (pairs i, i + rd/2) of the first rd = cs.shape[-1] dims of x [T, heads, d] (fp32)."""
+    rd = cs.shape[-1]
+    if rd == 0:
+        return x
+    h = rd // 2
+    c, s = cs[:, None, :h], cs[:, None, h:]
+    u, v = x[..., :h], x[..., h:rd]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., rd:]], dim=-1)
+
+
 def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache,
-                          q_temp=None) -> None:
+                          q_temp=None, span="head", layout="interleaved") -> None:
     T = qkv.shape[0]
     if T == 0:
         return
     bs = k_cache.shape[2]
-    q = qkv[:, : H * dk].float().view(T, H, dk)
-    k = qkv[:, H * dk:(H + G) * dk].float().view(T, G, dk)
+    q = qkv[:, : H * dk].float()
+    k = qkv[:, H * dk:(H + G) * dk].float()
     v = qkv[:, (H + G) * dk:(H + G) * dk + G * dv].view(T, G, dv)
-    q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw
-    k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw
+    if span == "full":
+        q = (q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw).view(T, H, dk)
+        k = (k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw).view(T, G, dk)
+    else:
+        q, k = q.view(T, H, dk), k.view(T, G, dk)
+        q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qw
+        k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps) * kw
     if q_temp is not None and q_temp[1] > 0:
         steps = torch.div(positions.long() + 1, int(q_temp[1]), rounding_mode="floor")
         q = q * (1.0 + float(q_temp[0]) * torch.log(steps.float() + 1.0))[:, None, None]
     if cos_sin is not None:
         cs = cos_sin[positions.long()]
-        q, k = _rot_pairs(q, cs), _rot_pairs(k, cs)
+        rot = _rot_halves if layout == "half" else _rot_pairs
+        q, k = rot(q, cs), rot(k, cs)
     qkv[:, : H * dk] = q.reshape(T, H * dk).to(qkv.dtype)
     ok = slots >= 0
     if ok.any():
@@ -151,18 +168,28 @@ def qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk,
 
 
 def qknorm_rope_cache(qkv, positions, slots, qw, kw, eps: float, cos_sin, H: int, G: int, dk: int, dv: int,
-                      k_cache, v_cache, q_temp=None) -> None:
+                      k_cache, v_cache, q_temp=None, span: str = "head", layout: str = "interleaved") -> None:
     """Rows of ``qkv`` = [q: H*dk | k: G*dk | v: G*dv | ...]: per-head RMS norm (weights ``qw`` /
     ``kw`` [dk], eps inside the root) and interleaved rotary (``cos_sin`` [max_pos, rd], or None)
     of q in place and of k into ``k_cache`` [NB, G, bs, dk]; v into ``v_cache`` [NB, G, bs, dv]
     at ``slots`` (-1: not written).  ``q_temp`` = (coef, every): the normalised q of a row at
-    position p is also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)."""
+    position p is also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).
+    ``span`` "full": the RMS runs over the whole q (and the whole k) projection of a row instead of
+    per head, with weights ``qw`` [H*dk] / ``kw`` [G*dk].  ``layout`` "half": rotary pairs are
+    (i, i + rd/2) inside a head instead of (2i, 2i+1)."""
     qt = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
     if _native(qkv):
-        _call("qknorm_rope_cache", qkv, positions, slots, qw, kw, float(eps), cos_sin, H, G, dk, dv, k_cache, v_cache,
-              qt[0], qt[1])
+        if span == "head" and layout == "interleaved":
+            _call("qknorm_rope_cache", qkv, positions, slots, qw, kw, float(eps), cos_sin, H, G, dk, dv, k_cache,
+                  v_cache, qt[0], qt[1])
+        else:
+            if qt[1]:
+                raise ValueError("qknorm_rope_cache: a query temperature needs span='head', layout='interleaved'")
+            _call("qk_prep", qkv, positions, slots, qw, kw, float(eps), cos_sin, H, G, dk, dv, k_cache, v_cache,
+                  span == "full", layout == "half")
     else:
-        qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache, qt)
+        qknorm_rope_cache_ref(qkv, positions, slots, qw, kw, eps, cos_sin, H, G, dk, dv, k_cache, v_cache, qt, span,
+                              layout)
 
 
 # ----------------------------------------------------------------------------
@@ -181,7 +208,7 @@ def distance_bias_table(rel: torch.Tensor, far: float) -> torch.Tensor:
 
 
 def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate=None,
-                         dist_bias=None, window=0):
+                         dist_bias=None, window=0, softcap=0.0, sinks=None):
     T = q.shape[0]
     bs, dk, dv = k_cache.shape[2], k_cache.shape[3], v_cache.shape[3]
     out = torch.zeros(T, H * dv, dtype=q.dtype, device=q.device)
@@ -205,7 +232,15 @@ def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, position
         if dist_bias is not None:
             d = (p - keys).clamp(max=dist_bias.shape[0] - 1)
             s = s + dist_bias[d].t().reshape(G, H // G, -1)
-        o = torch.einsum("ghn,ngd->ghd", torch.softmax(s, dim=-1), v).reshape(H * dv)
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        if sinks is not None:
+            # the sink is one more logit in the denominator; it has no value
+            s = torch.cat([s, sinks.float().reshape(G, H // G, 1)], dim=-1)
+            pr = torch.softmax(s, dim=-1)[..., :-1]
+        else:
+            pr = torch.softmax(s, dim=-1)
+        o = torch.einsum("ghn,ngd->ghd", pr, v).reshape(H * dv)
         if gate is not None:
             o = o * torch.sigmoid(gate[t, : H * dv].float())
         out[t] = o.to(q.dtype)
@@ -213,20 +248,22 @@ def masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, position
 
 
 def masked_attn_rows(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H: int, G: int, scale: float,
-                     mask: int = 0, gate=None, out=None, dist_bias=None) -> torch.Tensor:
+                     mask: int = 0, gate=None, out=None, dist_bias=None, softcap: float = 0.0, sinks=None) -> torch.Tensor:
     """Softmax attention of each row of ``q`` (position ``positions[t]``) over keys
     [floor(p / mask) * mask, p] of its sequence (``mask`` 0: [0, p]) read from the paged cache;
     rows map to ``block_tables`` rows through ``cu_seqlens`` (None: row i <-> table row i).
     ``gate``: the output is multiplied by sigmoid(gate) element by element.  ``dist_bias``
-    [n, H] fp32: added to the scaled score of a key at distance d = p - j, row min(d, n - 1)."""
+    [n, H] fp32: added to the scaled score of a key at distance d = p - j, row min(d, n - 1).
+    ``softcap`` > 0: the (scaled, biased) score s becomes softcap * tanh(s / softcap).  ``sinks`` [H] fp32:
+    exp(sinks[h]) joins head h's softmax denominator (a logit without a key or a value)."""
     if _native(q):
         if out is None:
             out = torch.empty(q.shape[0], H * v_cache.shape[3], dtype=q.dtype, device=q.device)
         _call("masked_attn_rows", out, q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, float(scale),
-              int(mask), gate, dist_bias)
+              int(mask), gate, dist_bias, float(softcap), sinks)
         return out
     r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens, positions, H, G, scale, mask, gate,
-                             dist_bias)
+                             dist_bias, 0, softcap, sinks)
     if out is not None:
         out.copy_(r)
         return out
@@ -247,11 +284,13 @@ def masked_prefill_available() -> bool:
 
 
 def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, nh, nkv, scale,
-                         mask: int = 0, gate=None, tiles=None, out=None, dist_bias=None, window: int = 0) -> torch.Tensor:
+                         mask: int = 0, gate=None, tiles=None, out=None, dist_bias=None, window: int = 0,
+                         softcap: float = 0.0, sinks=None) -> torch.Tensor:
     """``paged_prefill`` with a block mask — a query at position p sees keys
     [floor(p / mask) * mask, p] (``mask`` 0: all keys up to p) — or a sliding window (``window`` > 0
     with ``mask`` 0: keys [max(0, p - window + 1), p]) and an optional sigmoid output
     gate (out *= sigmoid(gate)) and an optional distance bias (``dist_bias`` as in
+    ``masked_attn_rows``), an optional score soft cap and per-head sink logits (``softcap`` / ``sinks``, as in
     ``masked_attn_rows``).  bf16, key size == value size in {64, 128} on the GPU
     (dgi/csrc/mix/masked_prefill.hip); the row-wise reference elsewhere."""
     from dgi import ops
@@ -265,13 +304,14 @@ def paged_prefill_masked(q, k_cache, v_cache, block_tables, cu_seqlens_q, contex
         if mask and window:
             raise ValueError("paged_prefill_masked: a block mask or a window, not both")
         _call("paged_prefill_masked", out, q, k_cache, v_cache, block_tables, cu_seqlens_q, context_lens, tiles,
-              nh, nkv, float(scale), int(mask) if mask else -int(window), gate, dist_bias)      # the kernel takes a window as a negative mask
+              nh, nkv, float(scale), int(mask) if mask else -int(window), gate, dist_bias,      # the kernel takes a window as a negative mask
+              float(softcap), sinks)
         return out
     cu = cu_seqlens_q.tolist()
     pos = torch.cat([torch.arange(int(context_lens[b]) - (cu[b + 1] - cu[b]), int(context_lens[b]), dtype=torch.int32)
                      for b in range(len(cu) - 1)]) if len(cu) > 1 else torch.zeros(0, dtype=torch.int32)
     r = masked_attn_rows_ref(q, k_cache, v_cache, block_tables, cu_seqlens_q, pos.to(q.device), nh, nkv, scale,
-                             mask, gate, dist_bias, window)
+                             mask, gate, dist_bias, window, softcap, sinks)
     if out is not None:
         out.copy_(r)
         return out

@@ -75,6 +75,10 @@ def glu_rows(gu: torch.Tensor, act: str = "silu", limit: float = 0.0, alpha: flo
 
 
 def moe_route_ref(logits, correction, top, score="softmax"):
+    if score == "top_softmax":
+        lf = logits.float()
+        idx = torch.sort(lf, dim=-1, descending=True, stable=True).indices[:, :top]
+        return idx.to(torch.int32), torch.softmax(torch.gather(lf, 1, idx), -1)
     s = torch.softmax(logits.float(), -1) if score == "softmax" else torch.sigmoid(logits.float())
     pick = s if correction is None else s + correction
     idx = torch.sort(pick, dim=-1, descending=True, stable=True).indices[:, :top]      # ties: the lowest index first
@@ -85,12 +89,15 @@ def moe_route(logits: torch.Tensor, correction, top: int, score: str = "softmax"
     """fp32 ``logits`` [T, R] -> (routes [T, top] int32 ordered by falling s + correction,
     weights [T, top] fp32 = the plain scores of those routes); s = softmax over the routes, or
     sigmoid of each (``score="sigmoid"``); ``correction`` None: the choice is by s alone.  Ties
-    go to the lowest index."""
+    go to the lowest index.  ``score="top_softmax"``: the ``top`` largest logits are taken and the
+    weights are the softmax over those alone (no ``correction``)."""
     if _native(logits):
         T = logits.shape[0]
         idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
         w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-        _call("moe_route", idx, w, logits, correction, 1 if score == "sigmoid" else 0)
+        if score == "top_softmax" and correction is not None:
+            raise ValueError("moe_route: top_softmax takes no selection bias")
+        _call("moe_route", idx, w, logits, correction, {"softmax": 0, "sigmoid": 1, "top_softmax": 2}[score])
         return idx, w
     return moe_route_ref(logits, correction, top, score)
 
