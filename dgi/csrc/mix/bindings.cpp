@@ -24,12 +24,13 @@ int dgi_qknorm_rope_cache(void* qkv, int is_f32, int T, int stride, const int* p
 int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                          int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H, int G,
                          int dk, int dv, int block_size, float scale, int mask, const void* gate, int gate_stride,
-                         void* out, int out_stride, int is_f32, const float* dist_bias, int n_dist, hipStream_t s);
+                         void* out, int out_stride, int is_f32, const float* dist_bias, int n_dist, float softcap,
+                         const float* sinks, hipStream_t s);
 int dgi_paged_prefill_masked(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                              const int* block_tables, int bt_stride, const int* cu_seqlens_q, const int* context_lens,
                              const int* tiles, int n_tiles, void* out, int out_stride, int nh, int nkv, int hd,
                              int block_size, float scale, int mask, const void* gate, int gate_stride,
-                             const float* dist_bias, int n_dist, hipStream_t s);
+                             const float* dist_bias, int n_dist, float softcap, const float* sinks, hipStream_t s);
 int dgi_glu_clamped(const void* gu, int gu_stride, void* out, int is_f32, int T, int I, float limit, float alpha,
                     hipStream_t s);
 int dgi_scale_softcap(const void* x, int x_stride, float* out, int is_f32, int T, int V, float scale, float cap,
@@ -55,7 +56,23 @@ int dgi_moe_route(int* idx, float* wts, const float* logits, int l_stride, const
 int dgi_glu_rows(void* out, const void* gu, int gu_stride, int rows, int I, int kind, float limit, float alpha,
                  const float* row_scale, int is_f32, hipStream_t s);
 int dgi_stream_add_norm(float* x, int T, int W, const void* y, int y_stride, int y_f32, const float* post_w,
-                        const float* next_w, float eps, void* out, int out_f32, hipStream_t s);
+                        const float* next_w, float eps, void* out, int out_f32, const void* y2, int y2_stride, int y2_f32,
+                        hipStream_t s);
+int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, const void* k, int k_stride, const void* v,
+                    int v_stride, int in_f32, const float* aux1, int aux1_stride, const float* aux2, int aux2_stride,
+                    const float* par1, const float* par2, float* state, float* norm, float* mx, const int* positions,
+                    const int* seq_row0, const int* seq_slots, int n_seq, int H, int G, int dk, int dv, float cap,
+                    int r_sel, hipStream_t st);
+int dgi_token_shift(void* out, int out_f32, const void* h, int h_f32, int h_stride, const float* mu, int nmix, float* tail,
+                    const int* positions, const int* row_seq, const int* seq_row0, const int* seq_slots, int n_seq, int T,
+                    int W, hipStream_t st);
+int dgi_head_norm_gate(void* out, int out_f32, const float* y, const void* z, int z_f32, int z_stride, const float* w,
+                       int wlen, int T, int H, int dv, float eps, int sigmoid_gate, hipStream_t st);
+int dgi_rms_pair_mean(float* out, const void* a, int a_stride, const void* b, int b_stride, int in_f32, const float* wa,
+                      const float* wb, int T, int W, float eps, hipStream_t st);
+int dgi_qk_prep(void* qkv, int is_f32, int T, int stride, const int* positions, const int* slots, const float* qw,
+                const float* kw, float eps, const float* cos_sin, int rd, int H, int G, int dk, int dv, void* k_cache,
+                void* v_cache, int block_size, int full, int half, hipStream_t s);
 int dgi_latent_prep(const void* proj, int stride, int is_f32, int T, int q_rank, int kv_rank, int rot_dim,
                     const float* dq_w, const float* dkv_w, float eps, const int* positions, const int* slots,
                     const float* cos_sin, int dims, int interleaved, void* cq, void* cache, hipStream_t s);
@@ -185,10 +202,16 @@ void qknorm_rope_cache(at::Tensor qkv, const at::Tensor& positions, const at::Te
 void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
                       const at::Tensor& block_tables, const c10::optional<at::Tensor>& cu_seqlens,
                       const at::Tensor& positions, int64_t H, int64_t G, double scale, int64_t mask,
-                      const c10::optional<at::Tensor>& gate, const c10::optional<at::Tensor>& dist_bias) {
+                      const c10::optional<at::Tensor>& gate, const c10::optional<at::Tensor>& dist_bias, double softcap,
+                      const c10::optional<at::Tensor>& sinks) {
   const int f = act_kind(q, "q");
   check_rows(q, "q"); check_rows(out, "out");
   TORCH_CHECK(act_kind(out, "out") == f && act_kind(k_cache, "k_cache") == f && act_kind(v_cache, "v_cache") == f);
+  const float* sk = nullptr;
+  if (sinks.has_value()) {
+    check_f32(*sinks, "sinks", H);
+    sk = sinks->data_ptr<float>();
+  }
   TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4);
   check_i32(block_tables, "block_tables"); check_i32(positions, "positions");
   TORCH_CHECK(block_tables.dim() == 2);
@@ -224,7 +247,8 @@ void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_c
   check_rc(dgi_masked_attn_rows(q.data_ptr(), (int)q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
                                 block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu, n_seqs,
                                 positions.data_ptr<int>(), rows, (int)H, (int)G, dk, dv, (int)k_cache.size(2), (float)scale,
-                                (int)mask, gp, gs, out.data_ptr(), (int)out.stride(0), f, db, nd, cur_stream()),
+                                (int)mask, gp, gs, out.data_ptr(), (int)out.stride(0), f, db, nd, (float)softcap, sk,
+                                cur_stream()),
            "masked_attn_rows");
 }
 
@@ -233,7 +257,13 @@ void masked_attn_rows(at::Tensor out, const at::Tensor& q, const at::Tensor& k_c
 void paged_prefill_masked(at::Tensor out, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
                           const at::Tensor& block_tables, const at::Tensor& cu_seqlens_q, const at::Tensor& context_lens,
                           const at::Tensor& tiles, int64_t nh, int64_t nkv, double scale, int64_t mask,
-                          const c10::optional<at::Tensor>& gate, const c10::optional<at::Tensor>& dist_bias) {
+                          const c10::optional<at::Tensor>& gate, const c10::optional<at::Tensor>& dist_bias, double softcap,
+                          const c10::optional<at::Tensor>& sinks) {
+  const float* sk = nullptr;
+  if (sinks.has_value()) {
+    check_f32(*sinks, "sinks", nh);
+    sk = sinks->data_ptr<float>();
+  }
   TORCH_CHECK(act_kind(q, "q") == 0 && act_kind(out, "out") == 0 && act_kind(k_cache, "k_cache") == 0 &&
               act_kind(v_cache, "v_cache") == 0, "paged_prefill_masked: bfloat16 only");
   check_rows(q, "q"); check_rows(out, "out");
@@ -269,7 +299,7 @@ void paged_prefill_masked(at::Tensor out, const at::Tensor& q, const at::Tensor&
                                     block_tables.data_ptr<int>(), (int)block_tables.stride(0), cu_seqlens_q.data_ptr<int>(),
                                     context_lens.data_ptr<int>(), tiles.data_ptr<int>(), (int)tiles.size(0), out.data_ptr(),
                                     (int)out.stride(0), (int)nh, (int)nkv, hd, (int)k_cache.size(2), (float)scale, (int)mask,
-                                    gp, gs, dbp, ndist, cur_stream()), "paged_prefill_masked");
+                                    gp, gs, dbp, ndist, (float)softcap, sk, cur_stream()), "paged_prefill_masked");
 }
 
 void glu_clamped(at::Tensor out, const at::Tensor& gu, double limit, double alpha) {
@@ -516,7 +546,8 @@ void glu_rows(at::Tensor out, const at::Tensor& gu, int64_t kind, double limit, 
 
 // x [T, W] fp32 += y (unit-RMS normed and weighted if post_w); out = RMS norm of x times next_w (or x) in out's dtype
 void stream_add_norm(at::Tensor x, const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& post_w,
-                     const c10::optional<at::Tensor>& next_w, double eps, c10::optional<at::Tensor> out) {
+                     const c10::optional<at::Tensor>& next_w, double eps, c10::optional<at::Tensor> out,
+                     const c10::optional<at::Tensor>& y2) {
   check_f32(x, "x");
   TORCH_CHECK(x.dim() == 2);
   const int T = (int)x.size(0), W = (int)x.size(1);
@@ -536,8 +567,17 @@ void stream_add_norm(at::Tensor x, const c10::optional<at::Tensor>& y, const c10
     TORCH_CHECK(out->is_contiguous() && out->dim() == 2 && out->size(0) == T && out->size(1) == W);
     op = out->data_ptr();
   }
+  const void* y2p = nullptr;
+  int y2s = 0, y2f = 1;
+  if (y2.has_value()) {
+    TORCH_CHECK(y.has_value(), "stream_add_norm: y2 needs y");
+    y2f = act_kind(*y2, "y2");
+    check_rows(*y2, "y2");
+    TORCH_CHECK(y2->size(0) == T && y2->size(1) == W, "stream_add_norm: y2 must be [T, W]");
+    y2p = y2->data_ptr(); y2s = (int)y2->stride(0);
+  }
   check_rc(dgi_stream_add_norm(x.data_ptr<float>(), T, W, yp, ys, yf, f32p(post_w, "post_w", W), f32p(next_w, "next_w", W),
-                               (float)eps, op, of, cur_stream()), "stream_add_norm");
+                               (float)eps, op, of, y2p, y2s, y2f, cur_stream()), "stream_add_norm");
 }
 
 void latent_prep(at::Tensor cq, const at::Tensor& proj, int64_t q_rank, int64_t kv_rank, int64_t rot_dim,
@@ -678,6 +718,122 @@ void gelu_tanh(at::Tensor out, const at::Tensor& x, const c10::optional<at::Tens
            "gelu_tanh");
 }
 
+// q / k / v: 2-D row views (unit column stride) of bf16 or fp32 activations, all of one dtype; aux1 / aux2 fp32 row views
+void linear_scan(at::Tensor y, int64_t mode, const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
+                 const at::Tensor& aux1, const c10::optional<at::Tensor>& aux2, const c10::optional<at::Tensor>& par1,
+                 const c10::optional<at::Tensor>& par2, at::Tensor state, c10::optional<at::Tensor> norm,
+                 c10::optional<at::Tensor> mx, const at::Tensor& positions, const at::Tensor& seq_row0,
+                 const at::Tensor& seq_slots, int64_t H, int64_t G, int64_t dk, int64_t dv, double cap, int64_t r_sel) {
+  check_f32(y, "y"); check_f32(state, "state");
+  const int f = act_kind(q, "q");
+  TORCH_CHECK(act_kind(k, "k") == f && act_kind(v, "v") == f, "linear_scan: q, k, v must share a dtype");
+  check_rows(q, "q"); check_rows(k, "k"); check_rows(v, "v"); check_rows(aux1, "aux1");
+  const int T = (int)q.size(0);
+  TORCH_CHECK(mode >= 0 && mode <= 2 && H > 0 && G > 0 && H % G == 0);
+  TORCH_CHECK(q.size(1) == G * dk && k.size(0) == T && k.size(1) == G * dk && v.size(0) == T && v.size(1) == H * dv,
+              "linear_scan: q / k must be [T, G*dk], v [T, H*dv]");
+  TORCH_CHECK(y.dim() == 2 && y.size(0) == T && y.size(1) == H * dv);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk && state.size(3) == dv,
+              "state must be [slots, H, dk, dv]");
+  TORCH_CHECK(aux1.is_cuda() && aux1.scalar_type() == at::kFloat && aux1.size(0) == T &&
+              aux1.size(1) == (mode == 0 ? H * dk : H), "linear_scan: aux1 shape");
+  const float* a2 = nullptr;
+  int a2s = 0;
+  if (aux2.has_value()) {
+    check_rows(*aux2, "aux2");
+    TORCH_CHECK(aux2->is_cuda() && aux2->scalar_type() == at::kFloat && aux2->size(0) == T && aux2->size(1) == H);
+    a2 = aux2->data_ptr<float>(); a2s = (int)aux2->stride(0);
+  }
+  const int64_t np = mode == 0 ? H * dk : H;
+  float *nrm = nullptr, *mxp = nullptr;
+  if (mode == 2) {
+    TORCH_CHECK(norm.has_value() && mx.has_value(), "linear_scan: the matrix memory needs its normaliser and maximum states");
+    check_f32(*norm, "norm"); check_f32(*mx, "mx");
+    TORCH_CHECK(norm->dim() == 3 && norm->size(0) == state.size(0) && norm->size(1) == H && norm->size(2) == dk);
+    TORCH_CHECK(mx->dim() == 2 && mx->size(0) == state.size(0) && mx->size(1) == H);
+    nrm = norm->data_ptr<float>(); mxp = mx->data_ptr<float>();
+  }
+  const int n_seq = (int)seq_slots.numel();
+  check_rc(dgi_linear_scan(y.data_ptr<float>(), (int)mode, q.data_ptr(), (int)q.stride(0), k.data_ptr(), (int)k.stride(0),
+                           v.data_ptr(), (int)v.stride(0), f, aux1.data_ptr<float>(), (int)aux1.stride(0), a2, a2s,
+                           f32p(par1, "par1", np), f32p(par2, "par2", np), state.data_ptr<float>(), nrm, mxp,
+                           i32p(positions, "positions", T), i32p(seq_row0, "seq_row0", n_seq + 1),
+                           i32p(seq_slots, "seq_slots"), n_seq, (int)H, (int)G, (int)dk, (int)dv, (float)cap, (int)r_sel,
+                           cur_stream()), "linear_scan");
+}
+
+// out [n, T, W] <- h + (previous row - h) * mu[n]; tail [slots, W] fp32 holds each sequence's last row
+void token_shift(at::Tensor out, const at::Tensor& h, const at::Tensor& mu, at::Tensor tail, const at::Tensor& positions,
+                 const at::Tensor& row_seq, const at::Tensor& seq_row0, const at::Tensor& seq_slots) {
+  const int hf = act_kind(h, "h"), of = act_kind(out, "out");
+  check_rows(h, "h");
+  const int T = (int)h.size(0), W = (int)h.size(1);
+  check_f32(mu, "mu"); check_f32(tail, "tail");
+  TORCH_CHECK(mu.dim() == 2 && mu.size(1) == W && tail.dim() == 2 && tail.size(1) == W);
+  const int nmix = (int)mu.size(0);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 3 && out.size(0) == nmix && out.size(1) == T && out.size(2) == W);
+  const int n_seq = (int)seq_slots.numel();
+  check_rc(dgi_token_shift(out.data_ptr(), of, h.data_ptr(), hf, (int)h.stride(0), mu.data_ptr<float>(), nmix,
+                           tail.data_ptr<float>(), i32p(positions, "positions", T), i32p(row_seq, "row_seq", T),
+                           i32p(seq_row0, "seq_row0", n_seq + 1), i32p(seq_slots, "seq_slots"), n_seq, T, W, cur_stream()),
+           "token_shift");
+}
+
+void head_norm_gate(at::Tensor out, const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t heads, double eps,
+                    int64_t sigmoid_gate) {
+  check_f32(y, "y"); check_f32(w, "w");
+  const int zf = act_kind(z, "z"), of = act_kind(out, "out");
+  check_rows(z, "z");
+  TORCH_CHECK(y.dim() == 2 && out.is_contiguous() && out.sizes() == y.sizes() && z.size(0) == y.size(0) && z.size(1) == y.size(1));
+  const int T = (int)y.size(0), C = (int)y.size(1);
+  TORCH_CHECK(heads > 0 && C % heads == 0 && w.numel() > 0 && C % w.numel() == 0, "head_norm_gate: sizes");
+  check_rc(dgi_head_norm_gate(out.data_ptr(), of, y.data_ptr<float>(), z.data_ptr(), zf, (int)z.stride(0), w.data_ptr<float>(),
+                              (int)w.numel(), T, (int)heads, C / (int)heads, (float)eps, (int)sigmoid_gate, cur_stream()),
+           "head_norm_gate");
+}
+
+void rms_pair_mean(at::Tensor out, const at::Tensor& a, const at::Tensor& b, const at::Tensor& wa, const at::Tensor& wb,
+                   double eps) {
+  check_f32(out, "out");
+  const int f = act_kind(a, "a");
+  TORCH_CHECK(act_kind(b, "b") == f);
+  check_rows(a, "a"); check_rows(b, "b");
+  const int T = (int)a.size(0), W = (int)a.size(1);
+  TORCH_CHECK(b.size(0) == T && b.size(1) == W && out.dim() == 2 && out.size(0) == T && out.size(1) == W);
+  check_f32(wa, "wa", W); check_f32(wb, "wb", W);
+  check_rc(dgi_rms_pair_mean(out.data_ptr<float>(), a.data_ptr(), (int)a.stride(0), b.data_ptr(), (int)b.stride(0), f,
+                             wa.data_ptr<float>(), wb.data_ptr<float>(), T, W, (float)eps, cur_stream()), "rms_pair_mean");
+}
+
+// qkv rows: [q: H*dk | k: G*dk | v: G*dv | ...]; full: norm over the whole q / k projection (weights [H*dk] / [G*dk])
+void qk_prep(at::Tensor qkv, const at::Tensor& positions, const at::Tensor& slots, const at::Tensor& qw, const at::Tensor& kw,
+             double eps, const c10::optional<at::Tensor>& cos_sin, int64_t H, int64_t G, int64_t dk, int64_t dv,
+             at::Tensor k_cache, at::Tensor v_cache, bool full, bool half) {
+  const int f = act_kind(qkv, "qkv");
+  check_rows(qkv, "qkv");
+  check_i32(positions, "positions"); check_i32(slots, "slots");
+  check_f32(qw, "qw", full ? H * dk : dk); check_f32(kw, "kw", full ? G * dk : dk);
+  const int T = (int)qkv.size(0);
+  TORCH_CHECK(positions.numel() == T && slots.numel() == T);
+  TORCH_CHECK(qkv.size(1) >= (H + G) * dk + G * dv, "qkv rows too short");
+  TORCH_CHECK(act_kind(k_cache, "k_cache") == f && act_kind(v_cache, "v_cache") == f);
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4);
+  TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == dk && v_cache.size(1) == G && v_cache.size(3) == dv &&
+              v_cache.size(0) == k_cache.size(0) && v_cache.size(2) == k_cache.size(2), "cache geometry");
+  int rd = 0;
+  const float* cs = nullptr;
+  if (cos_sin.has_value()) {
+    check_f32(*cos_sin, "cos_sin");
+    TORCH_CHECK(cos_sin->dim() == 2);
+    rd = (int)cos_sin->size(1);
+    cs = cos_sin->data_ptr<float>();
+  }
+  check_rc(dgi_qk_prep(qkv.data_ptr(), f, T, (int)qkv.stride(0), positions.data_ptr<int>(), slots.data_ptr<int>(),
+                       qw.data_ptr<float>(), kw.data_ptr<float>(), (float)eps, cs, rd, (int)H, (int)G, (int)dk, (int)dv,
+                       k_cache.data_ptr(), v_cache.data_ptr(), (int)k_cache.size(2), full ? 1 : 0, half ? 1 : 0, cur_stream()),
+           "qk_prep");
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(dgi, m) {
@@ -688,12 +844,21 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
   m.def("qknorm_rope_cache(Tensor(a!) qkv, Tensor positions, Tensor slots, Tensor qw, Tensor kw, float eps, "
         "Tensor? cos_sin, int H, int G, int dk, int dv, Tensor(b!) k_cache, Tensor(c!) v_cache, float qt_coef=0.0, "
         "int qt_every=0) -> ()");
+  m.def("linear_scan(Tensor(a!) y, int mode, Tensor q, Tensor k, Tensor v, Tensor aux1, Tensor? aux2, Tensor? par1, Tensor? par2, "
+        "Tensor(b!) state, Tensor(c!)? norm, Tensor(d!)? mx, Tensor positions, Tensor seq_row0, Tensor seq_slots, int H, int G, "
+        "int dk, int dv, float cap, int r_sel=0) -> ()");
+  m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) tail, Tensor positions, Tensor row_seq, Tensor seq_row0, "
+        "Tensor seq_slots) -> ()");
+  m.def("head_norm_gate(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int heads, float eps, int sigmoid_gate) -> ()");
+  m.def("rms_pair_mean(Tensor(a!) out, Tensor a, Tensor b, Tensor wa, Tensor wb, float eps) -> ()");
+  m.def("qk_prep(Tensor(a!) qkv, Tensor positions, Tensor slots, Tensor qw, Tensor kw, float eps, Tensor? cos_sin, int H, int G, "
+        "int dk, int dv, Tensor(b!) k_cache, Tensor(c!) v_cache, bool full, bool half) -> ()");
   m.def("masked_attn_rows(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
         "Tensor? cu_seqlens, Tensor positions, int H, int G, float scale, int mask, Tensor? gate, "
-        "Tensor? dist_bias=None) -> ()");
+        "Tensor? dist_bias=None, float softcap=0.0, Tensor? sinks=None) -> ()");
   m.def("paged_prefill_masked(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
         "Tensor cu_seqlens_q, Tensor context_lens, Tensor tiles, int nh, int nkv, float scale, int mask, "
-        "Tensor? gate, Tensor? dist_bias=None) -> ()");
+        "Tensor? gate, Tensor? dist_bias=None, float softcap=0.0, Tensor? sinks=None) -> ()");
   m.def("glu_clamped(Tensor(a!) out, Tensor gu, float limit, float alpha) -> ()");
   m.def("scale_softcap(Tensor(a!) out, Tensor x, float scale, float cap) -> ()");
   m.def("embed_streams(Tensor(a!) xs, Tensor ids, Tensor positions, Tensor row_seq, Tensor seq_row0, Tensor seq_slots, "
@@ -708,7 +873,8 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
   m.def("gated_group_norm(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int groups, float eps) -> ()");
   m.def("moe_route(Tensor(a!) idx, Tensor(b!) wts, Tensor logits, Tensor? correction, int sigmoid=0) -> ()");
   m.def("glu_rows(Tensor(a!) out, Tensor gu, int kind, float limit, float alpha, Tensor? row_scale) -> ()");
-  m.def("stream_add_norm(Tensor(a!) x, Tensor? y, Tensor? post_w, Tensor? next_w, float eps, Tensor(b!)? out) -> ()");
+  m.def("stream_add_norm(Tensor(a!) x, Tensor? y, Tensor? post_w, Tensor? next_w, float eps, Tensor(b!)? out, "
+        "Tensor? y2=None) -> ()");
   m.def("latent_prep(Tensor(a!) cq, Tensor proj, int q_rank, int kv_rank, int rot_dim, Tensor dq_w, Tensor? dkv_w, float eps, "
         "Tensor positions, Tensor slots, Tensor? cos_sin, bool interleaved, Tensor(b!)? cache) -> ()");
   m.def("latent_attn_rows(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor cache, Tensor block_tables, Tensor? cu_seqlens, "
@@ -729,6 +895,11 @@ TORCH_LIBRARY_IMPL(dgi, CUDA, m) {
   m.impl("dyt_add", &dyt_add);
   m.impl("embed_dyt", &embed_dyt);
   m.impl("qknorm_rope_cache", &qknorm_rope_cache);
+  m.impl("linear_scan", &linear_scan);
+  m.impl("token_shift", &token_shift);
+  m.impl("head_norm_gate", &head_norm_gate);
+  m.impl("rms_pair_mean", &rms_pair_mean);
+  m.impl("qk_prep", &qk_prep);
   m.impl("masked_attn_rows", &masked_attn_rows);
   m.impl("paged_prefill_masked", &paged_prefill_masked);
   m.impl("glu_clamped", &glu_clamped);

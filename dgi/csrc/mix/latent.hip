@@ -1,6 +1,7 @@
 // dgi/csrc/mix/latent.hip — row kernels of latent-attention models on an fp32 residual stream.
 //
-//   stream_add_norm   x += y   (or x += y / rms(y) * post_w)   and   out = x / rms(x) * next_w  (or out = x)
+//   stream_add_norm   x += y   (or x += y / rms(y) * post_w; or x += y + y2, two sublayers of one step)   and
+//                     out = x / rms(x) * next_w  (or out = x)
 //                     in one pass over the row: the residual add of one sublayer fused with the RMS
 //                     norm that feeds the next GEMM (the fused_add_rmsnorm of models whose stream is fp32)
 //   latent_prep       row = [query latent | key/value latent | key part | ...] from one fused GEMM:
@@ -63,11 +64,15 @@ template <typename TY, typename TO, int V>
 __global__ __launch_bounds__(NT) void stream_add_norm_kernel(float* __restrict__ x, int W, const TY* __restrict__ y,
                                                              int y_stride, const float* __restrict__ post_w,
                                                              const float* __restrict__ next_w, float eps,
-                                                             TO* __restrict__ out) {
+                                                             TO* __restrict__ out, const void* __restrict__ y2,
+                                                             int y2_stride, int y2_f32) {
   __shared__ float red[NT / 64];
   const int row = blockIdx.x;
   float* xr = x + (size_t)row * W;
   const TY* yr = y ? y + (size_t)row * y_stride : nullptr;
+  // second addend of the same step (bf16 or fp32, chosen at run time: uniform branches)
+  const float* y2f = (y2 && y2_f32) ? (const float*)y2 + (size_t)row * y2_stride : nullptr;
+  const uint16_t* y2h = (y2 && !y2_f32) ? (const uint16_t*)y2 + (size_t)row * y2_stride : nullptr;
   float xv[MAXV][V], yv[MAXV][V];
   float ssy = 0.f;
 #pragma unroll
@@ -95,7 +100,19 @@ __global__ __launch_bounds__(NT) void stream_add_norm_kernel(float* __restrict__
       const int c = (threadIdx.x + k * NT) * V;
       if (c < W) {
 #pragma unroll
-        for (int j = 0; j < V; ++j) xv[k][j] += post_w ? yv[k][j] * inv_y * post_w[c + j] : yv[k][j];
+        for (int j = 0; j < V; ++j) yv[k][j] = post_w ? yv[k][j] * inv_y * post_w[c + j] : yv[k][j];
+        if (y2f || y2h) {
+          float zv[V];
+          if constexpr (V == 4) {
+            if (y2f) ld4<float>(y2f + c, zv); else ld4<uint16_t>(y2h + c, zv);
+          } else {
+            zv[0] = y2f ? y2f[c] : bf16_to_f32(y2h[c]);
+          }
+#pragma unroll
+          for (int j = 0; j < V; ++j) yv[k][j] += zv[j];
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) xv[k][j] += yv[k][j];
         if constexpr (V == 4) st4<float>(xr + c, xv[k]);
         else xr[c] = xv[k][0];
       }
@@ -312,15 +329,18 @@ __global__ __launch_bounds__(NT) void gelu_tanh_vec_kernel(T* __restrict__ out, 
 }  // namespace
 
 extern "C" int dgi_stream_add_norm(float* x, int T, int W, const void* y, int y_stride, int y_f32, const float* post_w,
-                                   const float* next_w, float eps, void* out, int out_f32, hipStream_t s) {
+                                   const float* next_w, float eps, void* out, int out_f32, const void* y2, int y2_stride,
+                                   int y2_f32, hipStream_t s) {
   if (T == 0 || W == 0) return 0;
   if (W > NT * 4 * MAXV) return -3;
-  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)out) & 15) == 0 &&
+  if (y2 && !y) return -5;
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && y2_stride % 4 == 0 &&
+                   (((uintptr_t)x | (uintptr_t)y | (uintptr_t)out | (uintptr_t)y2) & 15) == 0 &&
                    W >= NT * 4;       // narrow rows: one column per thread and chunk keeps every thread busy
 #define DGI_SAN(TY_, TO_)                                                                                              \
   do {                                                                                                                 \
-    if (vec) stream_add_norm_kernel<TY_, TO_, 4><<<T, NT, 0, s>>>(x, W, (const TY_*)y, y_stride, post_w, next_w, eps, (TO_*)out); \
-    else if (W <= NT * MAXV) stream_add_norm_kernel<TY_, TO_, 1><<<T, NT, 0, s>>>(x, W, (const TY_*)y, y_stride, post_w, next_w, eps, (TO_*)out); \
+    if (vec) stream_add_norm_kernel<TY_, TO_, 4><<<T, NT, 0, s>>>(x, W, (const TY_*)y, y_stride, post_w, next_w, eps, (TO_*)out, y2, y2_stride, y2_f32); \
+    else if (W <= NT * MAXV) stream_add_norm_kernel<TY_, TO_, 1><<<T, NT, 0, s>>>(x, W, (const TY_*)y, y_stride, post_w, next_w, eps, (TO_*)out, y2, y2_stride, y2_f32); \
     else return -4;                                                                                                    \
   } while (0)
   if (y_f32) { if (out_f32) DGI_SAN(float, float); else DGI_SAN(float, uint16_t); }

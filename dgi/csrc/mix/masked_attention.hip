@@ -17,6 +17,9 @@
 // Scores, the online softmax and the output accumulation are fp32; exp is the accurate expf.
 // Optional distance bias: dist_bias[min(p - j, n_dist - 1)][head] (fp32, one row per distance, the
 // last row for everything farther) is added to the scaled score of key j before the softmax.
+// Optional soft cap: the scaled (and biased) score s becomes softcap * tanh(s / softcap).
+// Optional sinks: exp(sinks[head]) joins the softmax denominator of that head (a logit that has no
+// key and no value; it is neither scaled nor capped).
 // Optional epilogue: out *= sigmoid(gate) element by element (the mixer's output gate, read
 // from the same fused projection row as q).
 //
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(64) void masked_attn_rows_kernel(
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu_seqlens, int n_seqs,
     const int* __restrict__ positions, int G, int dk, int dv, int bs, float scale, int mask,
     const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
-    const float* __restrict__ dist_bias, int n_dist) {
+    const float* __restrict__ dist_bias, int n_dist, float softcap, const float* __restrict__ sinks) {
   __shared__ float qs[MAXDK];
   __shared__ float ps[64];
   __shared__ long long vo[64];
@@ -116,6 +119,7 @@ __global__ __launch_bounds__(64) void masked_attn_rows_kernel(
       const long long slot = ((long long)blk * G + kvh) * bs + (key % bs);
       s = dot_row(qs, k_cache + slot * dk, dk) * scale;
       if (dist_bias) s += dist_bias[(size_t)min(pos - key, n_dist - 1) * H + head];
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       vbase = slot * dv;
     }
     const float m_new = fmaxf(m_run, wave_max(s));     // lane 0's key k0 is always visible: finite
@@ -139,7 +143,13 @@ __global__ __launch_bounds__(64) void masked_attn_rows_kernel(
       }
     }
   }
-  const float inv = 1.f / l_run;
+  float inv = 1.f / l_run;
+  if (sinks) {
+    // the sink logit joins the denominator only: out = o / (l + exp(sink - m)), with the larger of the two as reference
+    const float sk = sinks[head], m2 = fmaxf(m_run, sk);
+    const float f = expf(m_run - m2);
+    inv = f / (l_run * f + expf(sk - m2));
+  }
   T* op = out + (size_t)row * out_stride + (size_t)head * dv;
   const T* gp = gate ? gate + (size_t)row * gate_stride + (size_t)head * dv : nullptr;
 #pragma unroll
@@ -169,7 +179,7 @@ __global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu_seqlens, int n_seqs,
     const int* __restrict__ positions, int H, int dk, int dv, int bs, float scale, int mask,
     const T* __restrict__ gate, int gate_stride, T* __restrict__ out, int out_stride,
-    const float* __restrict__ dist_bias, int n_dist) {
+    const float* __restrict__ dist_bias, int n_dist, float softcap, const float* __restrict__ sinks) {
   constexpr int E = 16 / sizeof(T);
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int row = blockIdx.x, kvh = blockIdx.y, G = gridDim.y;
@@ -250,6 +260,7 @@ __global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
         if (ok) {
           s = sc[i] * scale;
           if (dist_bias) s += dist_bias[(size_t)min(pos - key, n_dist - 1) * H + kvh * r + i];
+          if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float m_new = fmaxf(m[i], wave_max(s));       // key k0 (lane 0) is visible: finite
         const float p = ok ? expf(s - m_new) : 0.f;
@@ -329,10 +340,11 @@ __global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
   __syncthreads();
   for (int idx = tid; idx < r * dv; idx += 64 * GNW) {
     const int i = idx / dv, d = idx - i * dv;
-    float M = -__builtin_inff();
+    const int head = kvh * r + i;
+    float M = sinks ? sinks[head] : -__builtin_inff();
 #pragma unroll
     for (int ww = 0; ww < GNW; ++ww) M = fmaxf(M, cm[ww * R + i]);
-    float L = 0.f, O = 0.f;
+    float L = sinks ? expf(sinks[head] - M) : 0.f, O = 0.f;      // the sink: one more term of the denominator
 #pragma unroll
     for (int ww = 0; ww < GNW; ++ww) {
       const float f = expf(cm[ww * R + i] - M);          // waves without a tile: exp(-inf) = 0
@@ -340,7 +352,6 @@ __global__ __launch_bounds__(64 * GNW) void masked_attn_group_kernel(
       O += co[((size_t)ww * R + i) * dv + d] * f;
     }
     float v = O / L;
-    const int head = kvh * r + i;
     if (gate) v *= 1.f / (1.f + expf(-ldf<T>(gate + (size_t)row * gate_stride + (size_t)head * dv + d)));
     stf<T>(out + (size_t)row * out_stride + (size_t)head * dv + d, v);
   }
@@ -350,12 +361,13 @@ template <typename T, int R, int VP>
 int launch_group(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                  int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions, int rows, int H, int G, int dk,
                  int dv, int bs, float scale, int mask, const void* gate, int gate_stride, void* out, int out_stride,
-                 const float* dist_bias, int n_dist, hipStream_t s) {
+                 const float* dist_bias, int n_dist, float softcap, const float* sinks, hipStream_t s) {
   const size_t lds = (size_t)(R * dk + GNW * R * 64 + GNW * 64 + 2 * GNW * R + GNW * R * dv) * 4;
   if (lds > 64 * 1024) return -1;
   masked_attn_group_kernel<T, R, VP><<<dim3(rows, G), 64 * GNW, lds, s>>>(
       (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, block_tables, bt_stride, cu_seqlens, n_seqs,
-      positions, H, dk, dv, bs, scale, mask, (const T*)gate, gate_stride, (T*)out, out_stride, dist_bias, n_dist);
+      positions, H, dk, dv, bs, scale, mask, (const T*)gate, gate_stride, (T*)out, out_stride, dist_bias, n_dist,
+      softcap, sinks);
   return 0;
 }
 
@@ -363,11 +375,12 @@ template <typename T>
 int dispatch_group(int r, int vpn, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                    const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs, const int* positions,
                    int rows, int H, int G, int dk, int dv, int bs, float scale, int mask, const void* gate,
-                   int gate_stride, void* out, int out_stride, const float* dist_bias, int n_dist, hipStream_t s) {
+                   int gate_stride, void* out, int out_stride, const float* dist_bias, int n_dist, float softcap,
+                   const float* sinks, hipStream_t s) {
 #define DGI_GRP(RV, VPV)                                                                                       \
   return launch_group<T, RV, VPV>(q, q_stride, k_cache, v_cache, block_tables, bt_stride, cu_seqlens, n_seqs, \
                                   positions, rows, H, G, dk, dv, bs, scale, mask, gate, gate_stride, out, out_stride, dist_bias, \
-                                  n_dist, s)
+                                  n_dist, softcap, sinks, s)
   if (vpn == 1) {
     if (r == 1) DGI_GRP(1, 1);
     if (r == 2) DGI_GRP(2, 1);
@@ -389,7 +402,8 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
                                     const int* block_tables, int bt_stride, const int* cu_seqlens, int n_seqs,
                                     const int* positions, int rows, int H, int G, int dk, int dv, int block_size,
                                     float scale, int mask, const void* gate, int gate_stride, void* out,
-                                    int out_stride, int is_f32, const float* dist_bias, int n_dist, hipStream_t s) {
+                                    int out_stride, int is_f32, const float* dist_bias, int n_dist, float softcap,
+                                    const float* sinks, hipStream_t s) {
   if (rows == 0) return 0;
   if (G <= 0 || H % G) return -2;
   if (dk > MAXDK || dv > 64 * MAXC || dk <= 0 || dv <= 0) return -3;
@@ -403,10 +417,11 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
     if (dk % E == 0 && dv % E == 0 && r <= 8 && vpn <= 2 && r * dv <= 1024 && aligned && G <= 65535) {
       const int rc = is_f32 ? dispatch_group<float>(r, vpn, q, q_stride, k_cache, v_cache, block_tables, bt_stride, cu_seqlens,
                                                     n_seqs, positions, rows, H, G, dk, dv, block_size, scale, mask, gate,
-                                                    gate_stride, out, out_stride, dist_bias, n_dist, s)
+                                                    gate_stride, out, out_stride, dist_bias, n_dist, softcap, sinks, s)
                             : dispatch_group<uint16_t>(r, vpn, q, q_stride, k_cache, v_cache, block_tables, bt_stride,
                                                        cu_seqlens, n_seqs, positions, rows, H, G, dk, dv, block_size, scale,
-                                                       mask, gate, gate_stride, out, out_stride, dist_bias, n_dist, s);
+                                                       mask, gate, gate_stride, out, out_stride, dist_bias, n_dist, softcap,
+                                                       sinks, s);
       if (rc == 0) {
         DGI_CHECK_LAUNCH();
         return 0;
@@ -418,12 +433,12 @@ extern "C" int dgi_masked_attn_rows(const void* q, int q_stride, const void* k_c
     masked_attn_rows_kernel<float><<<grid, 64, 0, s>>>(
         (const float*)q, q_stride, (const float*)k_cache, (const float*)v_cache, block_tables, bt_stride, cu_seqlens,
         n_seqs, positions, G, dk, dv, block_size, scale, mask, (const float*)gate, gate_stride, (float*)out, out_stride,
-        dist_bias, n_dist);
+        dist_bias, n_dist, softcap, sinks);
   else
     masked_attn_rows_kernel<uint16_t><<<grid, 64, 0, s>>>(
         (const uint16_t*)q, q_stride, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_tables, bt_stride,
         cu_seqlens, n_seqs, positions, G, dk, dv, block_size, scale, mask, (const uint16_t*)gate, gate_stride,
-        (uint16_t*)out, out_stride, dist_bias, n_dist);
+        (uint16_t*)out, out_stride, dist_bias, n_dist, softcap, sinks);
   DGI_CHECK_LAUNCH();
   return 0;
 }

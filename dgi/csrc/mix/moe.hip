@@ -2,7 +2,8 @@
 // small steps, and the combine of sorted-segment expert outputs for large ones.
 //
 //   moe_route         one wave per token: s = softmax(logits) over all R routes (fp32) or sigmoid of each, the
-//                     `top` routes with the largest s + correction (ties: lowest index), weights = s of those
+//                     `top` routes with the largest s + correction (ties: lowest index), weights = s of those;
+//                     mode 2: the `top` largest logits, weights = softmax over those alone
 //   silu_mul          silu(g) * u over fused [gate | up] rows
 //   glu_rows          the expert activation with an optional per-row factor on gate and up first (a route
 //                     weight on the expert's input, applied after the linear projections) and the clamped
@@ -58,6 +59,7 @@ constexpr int MAXR = 8;      // routes per lane: R <= 512
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, float* __restrict__ wts,
                                                        const float* __restrict__ logits, int l_stride,
                                                        const float* __restrict__ corr, int R, int top, int sigmoid) {
+  __shared__ float wsel[64 * MAXR];      // the chosen routes' weights, in order of choice
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* lp = logits + (size_t)t * l_stride;
   float s[MAXR], c[MAXR];
@@ -73,17 +75,28 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, fl
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
     const int r = lane + 64 * i;
-    if (sigmoid) s[i] = r < R ? 1.f / (1.f + expf(-s[i])) : 0.f;     // independent scores
+    if (sigmoid == 1) s[i] = r < R ? 1.f / (1.f + expf(-s[i])) : 0.f;     // independent scores
     else s[i] = r < R ? expf(s[i] - m) : 0.f;
     sum += s[i];
   }
-  const float inv = sigmoid ? 1.f : 1.f / wave_sum(sum);
+  const float inv = sigmoid == 1 ? 1.f : 1.f / wave_sum(sum);
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
     const int r = lane + 64 * i;
     s[i] *= inv;
     c[i] = r < R ? s[i] + (corr ? corr[r] : 0.f) : -__builtin_inff();
   }
+  if (sigmoid == 2) {
+    // choice by the logits themselves, weights exp(z - max) over the chosen ones, normalised below; the first
+    // pick is the row maximum, so every chosen term is exp of a non-positive number and the first is 1
+#pragma unroll
+    for (int i = 0; i < MAXR; ++i) {
+      const int r = lane + 64 * i;
+      c[i] = r < R ? lp[r] : -__builtin_inff();
+      s[i] = r < R ? expf(lp[r] - m) : 0.f;
+    }
+  }
+  float chosen = 0.f;
   for (int k = 0; k < top; ++k) {
     float bv = -__builtin_inff();
     int bi = 1 << 30;
@@ -102,11 +115,16 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ idx, fl
     for (int i = 0; i < MAXR; ++i) {
       if (lane + 64 * i == bi) {
         idx[(size_t)t * top + k] = bi;
-        wts[(size_t)t * top + k] = s[i];
+        wsel[k] = s[i];
+        chosen += s[i];
         c[i] = -__builtin_inff();
       }
     }
   }
+  chosen = wave_sum(chosen);              // each pick was added by the one lane that owns it
+  __syncthreads();
+  const float norm = sigmoid == 2 ? 1.f / chosen : 1.f;
+  for (int k = lane; k < top; k += 64) wts[(size_t)t * top + k] = wsel[k] * norm;
 }
 
 template <typename T> __device__ __forceinline__ void st4(T* p, const float* f);

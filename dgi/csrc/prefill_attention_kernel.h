@@ -9,6 +9,8 @@
 //     tile is "interior" (no per-element mask) only when it lies inside the block of the
 //     wave's last row;
 //   * an output gate: out *= sigmoid(gate) element by element in the epilogue (fp32).
+// With MASKED, softcap > 0 caps the scaled (and biased) score s at softcap * tanh(s / softcap), and sinks
+// (one fp32 logit per head) adds exp(sink) to the softmax denominator in the epilogue.
 // BIAS adds a learned distance bias to the scores before the mask: dist_bias[min(p - j, n_dist - 1)][head]
 // (fp32, natural score units; the kernel works in raw q.k units, hence inv_scale = 1 / scale).
 #pragma once
@@ -37,6 +39,9 @@ __device__ __forceinline__ int v_off(int row, int ch) {
 
 constexpr int KT = 64;  // keys per tile
 
+// 1 / scale from scale * log2(e)
+__device__ __forceinline__ float inv_scale_cap(float scale_log2) { return 1.4426950408889634f / scale_log2; }
+
 // NW waves x 32 query rows per workgroup (one K/V tile staging shared by all of them):
 // NW = 4 -> 128-row tiles, 2 workgroups per CU; NW = 8 -> 256-row tiles, 1 per CU
 // (same 2 waves per SIMD, half the K/V staging per query row).
@@ -53,7 +58,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
     const int* __restrict__ tiles, uint16_t* __restrict__ out, int out_stride, int nh, int nkv,
     int bs_log2, float scale_log2, const unsigned long long* __restrict__ tree_mask, int tree_n,
     int mask = 0, const uint16_t* __restrict__ gate = nullptr, int gate_stride = 0,
-    const float* __restrict__ dist_bias = nullptr, int n_dist = 0, float inv_scale = 0.f) {
+    const float* __restrict__ dist_bias = nullptr, int n_dist = 0, float inv_scale = 0.f,
+    float softcap = 0.f, const float* __restrict__ sinks = nullptr) {
   __shared__ __attribute__((aligned(16))) uint16_t lds[(DB ? 2 : 1) * 2 * KT * HD];
 
   const int b = tiles[2 * blockIdx.x];
@@ -262,6 +268,19 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
           }
       }
     }
+    if (MASKED && softcap > 0.f) {
+      // soft cap in natural score units, back to raw q.k units (the softmax below scales again):
+      // tanh(x) = 1 - 2 / (exp(2x) + 1) with the hardware exp2 / rcp
+      const float to_arg = scale_log2 * 2.f / softcap;             // raw -> 2 x log2(e)
+      const float back = softcap * inv_scale_cap(scale_log2);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = __builtin_amdgcn_exp2f(sc[kb][r] * to_arg);
+          sc[kb][r] = back * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
+        }
+    }
     // ---- online softmax; lane owns query lr, keys kb0 + 32kb + (r&3) + 8(r>>2) + 4hh.
     // Interior tiles (every key visible to every row of this wave, no tree rows) skip the
     // per-element mask; both kinds then share one exponent path.
@@ -373,6 +392,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void prefill_attn_kernel(
   }
 
   if (!row_valid) return;
+  if (MASKED && sinks) l_run += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - m_run);   // sink: denominator only
   const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
   uint16_t* op = out + (size_t)(q0 + my_row) * out_stride + head * HD;
 #pragma unroll

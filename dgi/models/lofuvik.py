@@ -195,6 +195,8 @@ class LofuvikModel:
                 fill(n, 0.1, 1.0)
             fill(L.side, W ** -0.5 * 2)
             fill(L.side_b, 0.3)
+            if L.spec.type == "delta":                 # the delta rule's gate projections have no bias
+                L.side_b[L.spec.mlp.routes if L.spec.mlp is not None else 0:].zero_()
             fill(L.gate_up, W ** -0.5)
             if L.down is not None:
                 fill(L.down, L.down.shape[-1] ** -0.5)

@@ -65,6 +65,18 @@ def rotate_half(x, cos, sin):
 
 
 # ------------------------------------------------------------------ mixers
+def wkv_core(r, k, v, dec, u):
+    """r, k, v, dec [T, H, D], u [H, D] -> o [T, H, D]; the bonus u replaces the state for the current token."""
+    T, H, D = r.shape
+    S = torch.zeros(H, D, D, dtype=F64)          # [head, key channel, value channel]
+    out = torch.zeros(T, H, D, dtype=F64)
+    for t in range(T):
+        kv = k[t, :, :, None] * v[t, :, None, :]
+        out[t] = torch.einsum("hkv,hk->hv", S + u[:, :, None] * kv, r[t])
+        S = dec[t, :, :, None] * S + kv
+    return out
+
+
 def wkv_mixer(w, p, m, h, eps):
     T = h.shape[0]
     H, D = int(m["heads"]), int(m["dim"])
@@ -78,13 +90,7 @@ def wkv_mixer(w, p, m, h, eps):
     v = lin(w[p + "v"], mixed("v")).view(T, H, D)
     gate = silu(lin(w[p + "g"], mixed("g")))
     dec = torch.exp(-torch.exp(lin(w[p + "w2"], torch.tanh(lin(w[p + "w1"], mixed("w")))) + w[p + "w0"])).view(T, H, D)
-    u = w[p + "u"].view(H, D)
-    S = torch.zeros(H, D, D, dtype=F64)          # [head, key channel, value channel]
-    out = torch.zeros(T, H, D, dtype=F64)
-    for t in range(T):
-        kv = k[t, :, :, None] * v[t, :, None, :]
-        out[t] = torch.einsum("hkv,hk->hv", S + u[:, :, None] * kv, r[t])
-        S = dec[t, :, :, None] * S + kv
+    out = wkv_core(r, k, v, dec, w[p + "u"].view(H, D))
     o = rms_unit(out, eps).reshape(T, H * D) * w[p + "norm"] * gate
     return lin(w[p + "o"], o)
 
@@ -100,18 +106,14 @@ def causal_conv_silu(x, taps_w):
     return silu(acc)
 
 
-def delta_mixer(w, p, m, h, eps):
-    T = h.shape[0]
-    H, G, D, V = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
-    q = causal_conv_silu(lin(w[p + "q"], h), w[p + "q.conv"]).view(T, G, D)
-    k = causal_conv_silu(lin(w[p + "k"], h), w[p + "k.conv"]).view(T, G, D)
-    v = causal_conv_silu(lin(w[p + "v"], h), w[p + "v.conv"]).view(T, H, V)
-    q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
-    k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
-    rep = H // G
-    q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
-    beta = torch.sigmoid(lin(w[p + "b"], h))
-    dec = torch.exp(-torch.exp(w[p + "A_log"]) * softplus(lin(w[p + "a"], h) + w[p + "dt_bias"]))
+def unit_vectors(x):
+    return x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6)
+
+
+def delta_core(q, k, v, beta, dec):
+    """q, k [T, H, D] (already unit vectors, q scaled), v [T, H, V], beta, dec [T, H] -> o [T, H, V]."""
+    T, H, D = q.shape
+    V = v.shape[2]
     S = torch.zeros(H, D, V, dtype=F64)
     out = torch.zeros(T, H, V, dtype=F64)
     for t in range(T):
@@ -119,8 +121,44 @@ def delta_mixer(w, p, m, h, eps):
         u = beta[t, :, None] * (v[t] - torch.einsum("hkv,hk->hv", S, k[t]))
         S = S + k[t, :, :, None] * u[:, None, :]
         out[t] = torch.einsum("hkv,hk->hv", S, q[t])
+    return out
+
+
+def delta_mixer(w, p, m, h, eps):
+    T = h.shape[0]
+    H, G, D, V = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+    q = causal_conv_silu(lin(w[p + "q"], h), w[p + "q.conv"]).view(T, G, D)
+    k = causal_conv_silu(lin(w[p + "k"], h), w[p + "k.conv"]).view(T, G, D)
+    v = causal_conv_silu(lin(w[p + "v"], h), w[p + "v.conv"]).view(T, H, V)
+    q = unit_vectors(q) * D ** -0.5
+    k = unit_vectors(k)
+    rep = H // G
+    q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(lin(w[p + "b"], h))
+    dec = torch.exp(-torch.exp(w[p + "A_log"]) * softplus(lin(w[p + "a"], h) + w[p + "dt_bias"]))
+    out = delta_core(q, k, v, beta, dec)
     o = (rms_unit(out, eps) * w[p + "norm"]).reshape(T, H * V) * silu(lin(w[p + "g"], h))
     return lin(w[p + "o"], o)
+
+
+def sink_attention_core(q, k, v, scale, cap, sink):
+    """q [T, H, D], k [T, G, D], v [T, G, V], sink [H] or None -> causal softmax attention [T, H, V]; the
+    sink is a logit of its own in the denominator (no key, no value, not scaled, not capped)."""
+    T, H, _ = q.shape
+    rep = H // k.shape[1]
+    k, v = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
+    s = torch.einsum("ihd,jhd->hij", q, k) * scale
+    if cap > 0:
+        s = cap * torch.tanh(s / cap)
+    s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), -math.inf)
+    top = s.max(-1).values
+    if sink is not None:
+        top = torch.maximum(top, sink[:, None])
+    e = torch.exp(s - top[..., None])
+    den = e.sum(-1, keepdim=True)
+    if sink is not None:
+        den = den + torch.exp(sink[:, None] - top)[..., None]
+    return torch.einsum("hij,jhd->ihd", e / den, v)
 
 
 def sink_attention(w, p, m, h, eps):
@@ -134,33 +172,22 @@ def sink_attention(w, p, m, h, eps):
     if rot and int(rot["dims"]) > 0:
         cos, sin = yarn_tables(rot, T)
         q, k = rotate_half(q, cos, sin), rotate_half(k, cos, sin)
-    rep = H // G
-    k, v = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
-    s = torch.einsum("ihd,jhd->hij", q, k) * float(m["scale"])
-    cap = float(m.get("softcap") or 0.0)
-    if cap > 0:
-        s = cap * torch.tanh(s / cap)
-    s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), -math.inf)
-    sink = w[p + "sink"]
-    top = torch.maximum(s.max(-1).values, sink[:, None])
-    e = torch.exp(s - top[..., None])
-    pr = e / (e.sum(-1, keepdim=True) + torch.exp(sink[:, None] - top)[..., None])
-    o = torch.einsum("hij,jhd->ihd", pr, v).reshape(T, H * V)
+    o = sink_attention_core(q, k, v, float(m["scale"]), float(m.get("softcap") or 0.0), w[p + "sink"]).reshape(T, H * V)
     return lin(w[p + "o"], o * torch.sigmoid(lin(w[p + "g"], h)))
 
 
-def mlstm_mixer(w, p, m, h, eps):
-    T = h.shape[0]
-    H, D, V = int(m["heads"]), int(m["dim"]), int(m["vdim"])
-    cap = float(m["gate_cap"])
-    q = lin(w[p + "q"], h).view(T, H, D) * D ** -0.5
-    k = lin(w[p + "k"], h).view(T, H, D)
-    v = lin(w[p + "v"], h).view(T, H, V)
-    ig = cap * torch.tanh((lin(w[p + "i"], h) + w[p + "i.b"]) / cap)
-    fg = torch.nn.functional.logsigmoid(cap * torch.tanh((lin(w[p + "f"], h) + w[p + "f.b"]) / cap))
+def capped_gates(i_raw, f_raw, cap):
+    """Log input gate and log forget gate from the projections (bias included)."""
+    return cap * torch.tanh(i_raw / cap), torch.nn.functional.logsigmoid(cap * torch.tanh(f_raw / cap))
+
+
+def mlstm_core(q, k, v, ig, fg):
+    """q (already scaled), k [T, H, D], v [T, H, V], log gates ig, fg [T, H] -> o [T, H, V]."""
+    T, H, D = q.shape
+    V = v.shape[2]
     S = torch.zeros(H, D, V, dtype=F64)
     n = torch.zeros(H, D, dtype=F64)
-    mx = torch.zeros(H, dtype=F64)
+    mx = torch.zeros(H, dtype=F64)               # the running maximum starts at 0
     out = torch.zeros(T, H, V, dtype=F64)
     for t in range(T):
         new = torch.maximum(fg[t] + mx, ig[t])
@@ -170,6 +197,18 @@ def mlstm_mixer(w, p, m, h, eps):
         mx = new
         den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-mx)) + 1e-6
         out[t] = torch.einsum("hkv,hk->hv", S, q[t]) / den[:, None]
+    return out
+
+
+def mlstm_mixer(w, p, m, h, eps):
+    T = h.shape[0]
+    H, D, V = int(m["heads"]), int(m["dim"]), int(m["vdim"])
+    cap = float(m["gate_cap"])
+    q = lin(w[p + "q"], h).view(T, H, D) * D ** -0.5
+    k = lin(w[p + "k"], h).view(T, H, D)
+    v = lin(w[p + "v"], h).view(T, H, V)
+    ig, fg = capped_gates(lin(w[p + "i"], h) + w[p + "i.b"], lin(w[p + "f"], h) + w[p + "f.b"], cap)
+    out = mlstm_core(q, k, v, ig, fg)
     o = rms_unit(out, eps).reshape(T, H * V) * w[p + "norm"] * torch.sigmoid(lin(w[p + "g"], h))
     return lin(w[p + "o"], o)
 
@@ -184,11 +223,15 @@ MIXERS = {"wkv": wkv_mixer, "delta": delta_mixer, "parallel": parallel_mixer}
 
 
 # ------------------------------------------------------------------ feed-forward
+def route_top(z, top):
+    """The `top` largest logits of every row and the softmax over those alone."""
+    val, idx = torch.topk(z, top, dim=-1)
+    return idx, torch.softmax(val, -1)
+
+
 def moe_ff(w, p, f, h):
     E, top = int(f["router"]["experts"]), int(f["router"]["top"])
-    z = lin(w[p + "router"], h) + w[p + "router.b"]
-    val, idx = torch.topk(z, top, dim=-1)
-    wt = torch.softmax(val, -1)
+    idx, wt = route_top(lin(w[p + "router"], h) + w[p + "router.b"], top)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(top):
