@@ -62,7 +62,8 @@ int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, const void*
                     int v_stride, int in_f32, const float* aux1, int aux1_stride, const float* aux2, int aux2_stride,
                     const float* par1, const float* par2, float* state, float* norm, float* mx, const int* positions,
                     const int* seq_row0, const int* seq_slots, int n_seq, int H, int G, int dk, int dv, float cap,
-                    int r_sel, hipStream_t st);
+                    int r_sel, float* norm_new, float* mx_new, hipStream_t st);
+int dgi_linear_scan_columns(int dk, int dv, int r_sel);
 int dgi_token_shift(void* out, int out_f32, const void* h, int h_f32, int h_stride, const float* mu, int nmix, float* tail,
                     const int* positions, const int* row_seq, const int* seq_row0, const int* seq_slots, int n_seq, int T,
                     int W, hipStream_t st);
@@ -754,12 +755,20 @@ void linear_scan(at::Tensor y, int64_t mode, const at::Tensor& q, const at::Tens
     nrm = norm->data_ptr<float>(); mxp = mx->data_ptr<float>();
   }
   const int n_seq = (int)seq_slots.numel();
+  // a matrix memory whose heads span several column blocks stages its new normaliser / maximum (committed by a second launch)
+  at::Tensor norm_new, mx_new;
+  float *nn = nullptr, *mn = nullptr;
+  if (mode == 2 && n_seq > 0 && dgi_linear_scan_columns((int)dk, (int)dv, (int)r_sel) < dv) {
+    norm_new = at::empty({n_seq, H, dk}, state.options());
+    mx_new = at::empty({n_seq, H}, state.options());
+    nn = norm_new.data_ptr<float>(); mn = mx_new.data_ptr<float>();
+  }
   check_rc(dgi_linear_scan(y.data_ptr<float>(), (int)mode, q.data_ptr(), (int)q.stride(0), k.data_ptr(), (int)k.stride(0),
                            v.data_ptr(), (int)v.stride(0), f, aux1.data_ptr<float>(), (int)aux1.stride(0), a2, a2s,
                            f32p(par1, "par1", np), f32p(par2, "par2", np), state.data_ptr<float>(), nrm, mxp,
                            i32p(positions, "positions", T), i32p(seq_row0, "seq_row0", n_seq + 1),
                            i32p(seq_slots, "seq_slots"), n_seq, (int)H, (int)G, (int)dk, (int)dv, (float)cap, (int)r_sel,
-                           cur_stream()), "linear_scan");
+                           nn, mn, cur_stream()), "linear_scan");
 }
 
 // out [n, T, W] <- h + (previous row - h) * mu[n]; tail [slots, W] fp32 holds each sequence's last row

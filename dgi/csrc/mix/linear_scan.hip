@@ -48,6 +48,7 @@ struct ScanArgs {
   float* state;                  // [slots, H, dk, dv]
   float* norm;                   // mlstm: [slots, H, dk]
   float* mx;                     // mlstm: [slots, H]
+  float *norm_new, *mx_new;      // mlstm with several column blocks per head: [n_seq, H, dk] / [n_seq, H] staging (see below)
   const int *positions, *seq_row0, *seq_slots;
   int H, G, dk, dv;
   int KS, CW, nwc, CB;           // key slices per wave, columns per wave, computing waves, columns per workgroup
@@ -234,10 +235,32 @@ __global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
     const int ch = s * R + i;
     if (col_ok && ch < dk) a.state[(sbase + ch) * dv + col] = S[i];
     if constexpr (MODE == MLSTM) {
-      if (cblk == 0 && wave == 0 && jl == 0 && ch < dk) a.norm[sbase + ch] = N[i];
+      // every column block of a head reads the normaliser and the maximum at its start and block 0 writes them at
+      // its end: with several blocks per head the new values go to a staging row and a second launch commits them,
+      // so a block that starts late still reads the old state
+      if (cblk == 0 && wave == 0 && jl == 0 && ch < dk) {
+        if (a.norm_new) a.norm_new[((size_t)seq * H + head) * dk + ch] = N[i];
+        else a.norm[sbase + ch] = N[i];
+      }
     }
   }
-  if (MODE == MLSTM && cblk == 0 && tid == 0) a.mx[(size_t)slot * H + head] = m_run;
+  if (MODE == MLSTM && cblk == 0 && tid == 0) {
+    if (a.mx_new) a.mx_new[(size_t)seq * H + head] = m_run;
+    else a.mx[(size_t)slot * H + head] = m_run;
+  }
+}
+
+// second launch of a matrix-memory scan whose heads span several column blocks: staged normaliser / maximum -> slots
+__global__ __launch_bounds__(256) void mlstm_commit_kernel(float* __restrict__ norm, float* __restrict__ mx,
+                                                           const float* __restrict__ norm_new,
+                                                           const float* __restrict__ mx_new,
+                                                           const int* __restrict__ seq_row0,
+                                                           const int* __restrict__ seq_slots, int H, int dk) {
+  const int seq = blockIdx.x;
+  if (seq_row0[seq + 1] <= seq_row0[seq]) return;
+  const size_t slot = (size_t)seq_slots[seq];
+  for (int i = threadIdx.x; i < H * dk; i += blockDim.x) norm[slot * H * dk + i] = norm_new[(size_t)seq * H * dk + i];
+  for (int i = threadIdx.x; i < H; i += blockDim.x) mx[slot * H + i] = mx_new[(size_t)seq * H + i];
 }
 
 template <int MODE, typename TI>
@@ -345,7 +368,7 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
                                int v_stride, int in_f32, const float* aux1, int aux1_stride, const float* aux2,
                                int aux2_stride, const float* par1, const float* par2, float* state, float* norm, float* mx,
                                const int* positions, const int* seq_row0, const int* seq_slots, int n_seq, int H, int G,
-                               int dk, int dv, float cap, int r_sel, hipStream_t st) {
+                               int dk, int dv, float cap, int r_sel, float* norm_new, float* mx_new, hipStream_t st) {
   if (n_seq == 0) return 0;
   if (mode < 0 || mode > 2 || H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0) return -2;
   if (dk > 512) return -3;
@@ -373,6 +396,10 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   if (nthreads > 512) return -5;
   const int nz = (dv + a.CB - 1) / a.CB;
   if (H > 65535 || nz > 65535) return -5;
+  const bool staged = mode == MLSTM && nz > 1;
+  if (staged && (!norm_new || !mx_new)) return -7;
+  a.norm_new = staged ? norm_new : nullptr;
+  a.mx_new = staged ? mx_new : nullptr;
   const dim3 grid(n_seq, H, nz);
   int rc;
 #define DGI_SCAN(M_)                                                                                      \
@@ -383,7 +410,23 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
 #undef DGI_SCAN
   if (rc) return rc;
   DGI_CHECK_LAUNCH();
+  if (staged) {
+    mlstm_commit_kernel<<<n_seq, 256, 0, st>>>(norm, mx, norm_new, mx_new, seq_row0, seq_slots, H, dk);
+    DGI_CHECK_LAUNCH();
+  }
   return 0;
+}
+
+// value columns one workgroup covers for this key size (the matrix memory stages its normaliser when dv exceeds it)
+extern "C" int dgi_linear_scan_columns(int dk, int dv, int r_sel) {
+  int R = r_sel > 0 ? r_sel : (dk <= 256 ? 16 : 32);
+  int KS = 1;
+  while (KS * R < dk) KS <<= 1;
+  if (KS > 64) return 0;
+  const int CW = 64 / KS;
+  int nwc = (dv + CW - 1) / CW;
+  if (nwc > 4) nwc = 4;
+  return nwc * CW;
 }
 
 extern "C" int dgi_token_shift(void* out, int out_f32, const void* h, int h_f32, int h_stride, const float* mu, int nmix,
