@@ -12,15 +12,17 @@
 //   head_norm_gate   per-head RMS norm of the recurrence's output, weight, silu / sigmoid gate
 //   rms_pair_mean    0.5 (a / rms(a) wa + b / rms(b) wb) over the model width
 //
-// linear_scan layout.  A workgroup owns (sequence, head, CB value columns).  Inside a wave, lane = s * CW + j:
-// column j of the wave's CW columns, key slice s of KS = 64 / CW slices; a thread keeps R consecutive key
-// channels of its column in registers (KS * R >= dk), so a token costs R fused multiply-adds per pass and the
-// sums over the key dimension finish with log2(KS) shuffles inside the wave — no barrier per token.
-// Tokens are staged TT at a time: every thread loads one key channel (and one value column) of each token into
-// registers while the previous tile is computed, the tile then goes to LDS (slices padded apart so the KS
-// broadcast reads of a wave hit different banks), per-token scalars (unit norms, decays, gates, the bonus dot
-// product, the stabiliser's running maximum) are computed once per token by one wave or one thread, and the
-// token loop reads LDS only.  Everything is fp32; q / k / v arrive as bf16 or fp32.
+// linear_scan layout.  A workgroup (256 threads) owns (sequence, head, CB value columns).  Inside a wave,
+// lane = j * KS + s: column j of the wave's CW = 64 / KS columns, key slice s of KS slices; a thread keeps R
+// consecutive key channels of its column in registers (KS * R >= dk), so a token costs R fused multiply-adds
+// per pass and the sums over the key dimension finish with log2(KS) xor-shuffles between ADJACENT lanes
+// (constant offsets below 16) — no barrier per token.  Tokens are staged TT (16) at a time: the tile is
+// loaded into registers, spread over all threads, while the previous tile is computed, then goes to LDS
+// (slices padded apart so the KS broadcast reads of a wave hit different banks; 16-byte reads).  Per-token
+// scalars are computed once per tile in parallel: unit norms / the bonus dot product by sixteen lanes per
+// token, decays and gates by one lane per token from gate inputs staged with the tile; only the stabiliser's
+// running maximum is a serial pass of one thread (adds and maxima; its exponentials are parallel again).
+// The token loop reads LDS only.  Everything is fp32; q / k / v arrive as bf16 or fp32.
 // A portion that starts at position 0 reads no state; the state is written back at the end of the portion.
 #include "../common.h"
 
@@ -58,8 +60,16 @@ struct ScanArgs {
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 __device__ __forceinline__ float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
-template <int MODE, typename TI, int R>
-__global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
+// R key channels per thread, KS key slices per value column (adjacent lanes: lane = column * KS + slice, so the sums
+// over the key dimension are log2(KS) xor-shuffles with constant offsets below 16), TT tokens per staged tile.
+template <int MODE, typename TI, int R, int KS, int TT>
+__global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
+  constexpr int CW = 64 / KS;                      // value columns per wave
+  constexpr int RP = R + 4;                        // padded key slice in LDS
+  constexpr int KP = KS * RP;                      // padded key row
+  constexpr int KSR = KS * R;                      // key channels covered (>= dk)
+  constexpr int NT = 256;
+  constexpr int NPF = (TT * KSR + NT - 1) / NT;    // staged key elements per thread and tile
   extern __shared__ __attribute__((aligned(16))) float sm[];
   const int seq = blockIdx.x, head = blockIdx.y, cblk = blockIdx.z;
   const int row0 = a.seq_row0[seq], n = a.seq_row0[seq + 1] - row0;
@@ -67,10 +77,10 @@ __global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
   const int p0 = a.positions[row0], slot = a.seq_slots[seq];
   const int dk = a.dk, dv = a.dv, H = a.H;
   const int kvh = head / (H / a.G);
-  const int KS = a.KS, CW = a.CW, CB = a.CB;
-  const int KP = KS * (R + 4);                     // padded key row in LDS
+  const int CB = a.CB;
+  const int NPV = (TT * CB + NT - 1) / NT;         // staged value elements per thread and tile (CB <= 256: at most TT)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int s = lane / CW, jl = lane - s * CW;
+  const int s = lane % KS, jl = lane / KS;
   const bool computes = wave < a.nwc;
   const int cl = wave * CW + jl;                   // column inside the workgroup
   const int col = cblk * CB + cl;
@@ -80,7 +90,9 @@ __global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
   float* sq = sk + TT * KP;
   float* sw = sq + TT * KP;                        // wkv only
   float* sv = sm + NV * TT * KP;                   // [TT][CB]
-  float* sc = sv + TT * CB;                        // [TT][4]
+  float* sc = sv + TT * CB;                        // [TT][4] per-token scalars
+  float* sg = sc + TT * 4;                         // [TT][4] raw gate inputs / stabiliser scratch
+  float* su = sg + TT * 4;                         // wkv: [KP] bonus
 
   float S[R], N[MODE == MLSTM ? R : 1];
   const size_t sbase = ((size_t)slot * H + head) * dk;
@@ -92,40 +104,65 @@ __global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
   }
   float m_run = 0.f;                               // mlstm stabiliser, carried by thread 0
   if (MODE == MLSTM && tid == 0 && p0 > 0) m_run = a.mx[(size_t)slot * H + head];
+  if constexpr (MODE == WKV) {
+    for (int ch = tid; ch < KSR; ch += NT) su[(ch / R) * RP + (ch % R)] = ch < dk ? a.par2[head * dk + ch] : 0.f;
+  }
 
-  // this thread's staged elements: key channel tid of every token, value column cblk * CB + tid
-  const bool ld_k = tid < dk, ld_pad = tid < KS * R, ld_v = tid < CB;
-  const bool v_ok = ld_v && cblk * CB + tid < dv;
-  const int kpi = (tid / R) * (R + 4) + (tid % R);
-  const TI* qp = (const TI*)a.q + (size_t)kvh * dk + tid;
-  const TI* kp = (const TI*)a.k + (size_t)kvh * dk + tid;
-  const TI* vp = (const TI*)a.v + (size_t)head * dv + cblk * CB + tid;
-  float w0 = 0.f;
-  if (MODE == WKV && ld_k) w0 = a.par1[head * dk + tid];
-  float pk[TT], pq[TT], pw[MODE == WKV ? TT : 1], pv[TT];
+  const TI* qp = (const TI*)a.q + (size_t)kvh * dk;
+  const TI* kp = (const TI*)a.k + (size_t)kvh * dk;
+  const TI* vp = (const TI*)a.v + (size_t)head * dv + cblk * CB;
+  float pk[NPF], pq[NPF], pw[MODE == WKV ? NPF : 1], pv[TT], pg1 = 0.f, pg2 = 0.f;
   auto load_tile = [&](int t0) {
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      const bool ok = t0 + tt < n;
+    for (int m = 0; m < NPF; ++m) {
+      const int e = tid + m * NT;
+      const int tt = e / KSR, ch = e % KSR;
+      const bool ok = tt < TT && t0 + tt < n && ch < dk;
       const size_t row = (size_t)(row0 + t0 + tt);
-      pk[tt] = (ok && ld_k) ? ldf<TI>(kp + row * a.k_stride) : 0.f;
-      pq[tt] = (ok && ld_k) ? ldf<TI>(qp + row * a.q_stride) : 0.f;
-      if constexpr (MODE == WKV) pw[tt] = (ok && ld_k) ? expf(-expf(a.aux1[row * a.aux1_stride + head * dk + tid] + w0)) : 0.f;
-      pv[tt] = (ok && v_ok) ? ldf<TI>(vp + row * a.v_stride) : 0.f;
+      pk[m] = ok ? ldf<TI>(kp + row * a.k_stride + ch) : 0.f;
+      pq[m] = ok ? ldf<TI>(qp + row * a.q_stride + ch) : 0.f;
+      if constexpr (MODE == WKV)
+        pw[m] = ok ? expf(-expf(a.aux1[row * a.aux1_stride + head * dk + ch] + a.par1[head * dk + ch])) : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < TT; ++m) {
+      pv[m] = 0.f;
+      if (m < NPV) {
+        const int e = tid + m * NT;
+        const int tt = e / CB, c = e - tt * CB;
+        if (tt < TT && t0 + tt < n && cblk * CB + c < dv) pv[m] = ldf<TI>(vp + (size_t)(row0 + t0 + tt) * a.v_stride + c);
+      }
+    }
+    if (MODE != WKV && tid < TT && t0 + tid < n) {
+      const size_t row = (size_t)(row0 + t0 + tid);
+      pg1 = a.aux1[row * a.aux1_stride + head];
+      pg2 = a.aux2[row * a.aux2_stride + head];
     }
   };
   auto store_tile = [&]() {
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      if (ld_pad) {
-        sk[tt * KP + kpi] = pk[tt];
-        sq[tt * KP + kpi] = pq[tt];
-        if constexpr (MODE == WKV) sw[tt * KP + kpi] = pw[tt];
+    for (int m = 0; m < NPF; ++m) {
+      const int e = tid + m * NT;
+      const int tt = e / KSR, ch = e % KSR;
+      if (tt < TT) {
+        const int o = tt * KP + (ch / R) * RP + (ch % R);
+        sk[o] = pk[m];
+        sq[o] = pq[m];
+        if constexpr (MODE == WKV) sw[o] = pw[m];
       }
-      if (ld_v) sv[tt * CB + tid] = pv[tt];
+    }
+#pragma unroll
+    for (int m = 0; m < TT; ++m) {
+      if (m < NPV) {
+        const int e = tid + m * NT;
+        if (e < TT * CB) sv[e] = pv[m];
+      }
+    }
+    if (MODE != WKV && tid < TT) {
+      sg[tid * 4] = pg1;
+      sg[tid * 4 + 1] = pg2;
     }
   };
-  const int nwaves = blockDim.x >> 6;
   const float qscale = 1.f / sqrtf((float)dk);
 
   load_tile(0);
@@ -134,42 +171,55 @@ __global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
     store_tile();
     __syncthreads();
     // ---- per-token scalars
-    if (MODE == MLSTM) {
+    if constexpr (MODE == MLSTM) {
+      // gates in parallel, the running maximum serially (adds and maxima only), the exponentials in parallel again
+      if (tid < nt) {
+        sg[tid * 4 + 2] = a.cap * tanhf(sg[tid * 4] / a.cap);
+        sg[tid * 4 + 3] = logsigmoid_f(a.cap * tanhf(sg[tid * 4 + 1] / a.cap));
+      }
+      __syncthreads();
       if (tid == 0) {
         for (int tt = 0; tt < nt; ++tt) {
-          const size_t row = (size_t)(row0 + t0 + tt);
-          const float ig = a.cap * tanhf(a.aux1[row * a.aux1_stride + head] / a.cap);
-          const float fg = logsigmoid_f(a.cap * tanhf(a.aux2[row * a.aux2_stride + head] / a.cap));
-          const float m_new = fmaxf(fg + m_run, ig);
-          sc[tt * 4 + 0] = expf(fg + m_run - m_new);
-          sc[tt * 4 + 1] = expf(ig - m_new);
-          sc[tt * 4 + 2] = expf(-m_new);
+          const float m_new = fmaxf(sg[tt * 4 + 3] + m_run, sg[tt * 4 + 2]);
+          sg[tt * 4] = m_run;                       // the maximum before this token
+          sg[tt * 4 + 1] = m_new;
           m_run = m_new;
         }
       }
+      __syncthreads();
+      if (tid < nt) {
+        const float m_old = sg[tid * 4], m_new = sg[tid * 4 + 1];
+        sc[tid * 4 + 0] = expf(sg[tid * 4 + 3] + m_old - m_new);
+        sc[tid * 4 + 1] = expf(sg[tid * 4 + 2] - m_new);
+        sc[tid * 4 + 2] = expf(-m_new);
+      }
     } else {
-      for (int tt = wave; tt < nt; tt += nwaves) {
+      // sixteen lanes per token: sums over the key channels, four shuffles inside the group
+      const int l = tid & 15;
+      for (int tt = tid >> 4; tt < nt; tt += NT / 16) {
         float r1 = 0.f, r2 = 0.f;
-        for (int i = lane; i < dk; i += 64) {
-          const int pi = (i / R) * (R + 4) + (i % R);
+        for (int i = l; i < dk; i += 16) {
+          const int pi = (i / R) * RP + (i % R);
           const float kv = sk[tt * KP + pi], qv = sq[tt * KP + pi];
           if (MODE == WKV) {
-            r1 += qv * kv * a.par2[head * dk + i];            // the bonus: sum_i r_i u_i k_i
+            r1 += qv * kv * su[pi];                 // the bonus: sum_i r_i u_i k_i
           } else {
             r1 += kv * kv;
             r2 += qv * qv;
           }
         }
-        r1 = wave_sum(r1);
-        if (MODE == DELTA) r2 = wave_sum(r2);
-        if (lane == 0) {
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+          r1 += __shfl_xor(r1, off, 64);
+          if (MODE == DELTA) r2 += __shfl_xor(r2, off, 64);
+        }
+        if (l == 0) {
           if (MODE == WKV) {
             sc[tt * 4] = r1;
           } else {
-            const size_t row = (size_t)(row0 + t0 + tt);
-            const float dt = softplus_f(a.aux2[row * a.aux2_stride + head] + a.par2[head]);
+            const float dt = softplus_f(sg[tt * 4 + 1] + a.par2[head]);
             sc[tt * 4 + 0] = expf(-expf(a.par1[head]) * dt);                        // decay
-            sc[tt * 4 + 1] = 1.f / (1.f + expf(-a.aux1[row * a.aux1_stride + head]));   // write strength
+            sc[tt * 4 + 1] = 1.f / (1.f + expf(-sg[tt * 4]));                       // write strength
             sc[tt * 4 + 2] = 1.f / sqrtf(r1 + 1e-6f);                               // 1 / |k|
             sc[tt * 4 + 3] = qscale / sqrtf(r2 + 1e-6f);                            // dk^-1/2 / |q|
           }
@@ -180,46 +230,67 @@ __global__ __launch_bounds__(512) void linear_scan_kernel(const ScanArgs a) {
     if (t0 + TT < n) load_tile(t0 + TT);             // in flight while this tile is computed
     if (computes) {
       for (int tt = 0; tt < nt; ++tt) {
-        const float* kk = sk + tt * KP + s * (R + 4);
-        const float* qq = sq + tt * KP + s * (R + 4);
+        const float4* kk = reinterpret_cast<const float4*>(sk + tt * KP + s * RP);
+        const float4* qq = reinterpret_cast<const float4*>(sq + tt * KP + s * RP);
         const float vj = sv[tt * CB + cl];
         float o;
         if constexpr (MODE == WKV) {
-          const float* ww = sw + tt * KP + s * (R + 4);
+          const float4* ww = reinterpret_cast<const float4*>(sw + tt * KP + s * RP);
           float acc = 0.f;
 #pragma unroll
-          for (int i = 0; i < R; ++i) acc += S[i] * qq[i];
+          for (int i = 0; i < R / 4; ++i) {
+            const float4 q4 = qq[i], k4 = kk[i], w4 = ww[i];
+            acc += S[4 * i] * q4.x + S[4 * i + 1] * q4.y + S[4 * i + 2] * q4.z + S[4 * i + 3] * q4.w;
+            S[4 * i] = w4.x * S[4 * i] + k4.x * vj;
+            S[4 * i + 1] = w4.y * S[4 * i + 1] + k4.y * vj;
+            S[4 * i + 2] = w4.z * S[4 * i + 2] + k4.z * vj;
+            S[4 * i + 3] = w4.w * S[4 * i + 3] + k4.w * vj;
+          }
 #pragma unroll
-          for (int i = 0; i < R; ++i) S[i] = ww[i] * S[i] + kk[i] * vj;
-          for (int off = CW; off < 64; off <<= 1) acc += __shfl_xor(acc, off, 64);
+          for (int off = 1; off < KS; off <<= 1) acc += __shfl_xor(acc, off, 64);
           o = acc + sc[tt * 4] * vj;
         } else if constexpr (MODE == DELTA) {
           const float g = sc[tt * 4], beta = sc[tt * 4 + 1], rk = sc[tt * 4 + 2], rq = sc[tt * 4 + 3];
           float pred = 0.f;
 #pragma unroll
-          for (int i = 0; i < R; ++i) pred += S[i] * kk[i];
-          for (int off = CW; off < 64; off <<= 1) pred += __shfl_xor(pred, off, 64);
+          for (int i = 0; i < R / 4; ++i) {
+            const float4 k4 = kk[i];
+            pred += S[4 * i] * k4.x + S[4 * i + 1] * k4.y + S[4 * i + 2] * k4.z + S[4 * i + 3] * k4.w;
+          }
+#pragma unroll
+          for (int off = 1; off < KS; off <<= 1) pred += __shfl_xor(pred, off, 64);
           const float ku = beta * (vj - pred * g * rk) * rk;
           float acc = 0.f;
 #pragma unroll
-          for (int i = 0; i < R; ++i) {
-            S[i] = g * S[i] + kk[i] * ku;
-            acc += S[i] * qq[i];
+          for (int i = 0; i < R / 4; ++i) {
+            const float4 k4 = kk[i], q4 = qq[i];
+            S[4 * i] = g * S[4 * i] + k4.x * ku;
+            S[4 * i + 1] = g * S[4 * i + 1] + k4.y * ku;
+            S[4 * i + 2] = g * S[4 * i + 2] + k4.z * ku;
+            S[4 * i + 3] = g * S[4 * i + 3] + k4.w * ku;
+            acc += S[4 * i] * q4.x + S[4 * i + 1] * q4.y + S[4 * i + 2] * q4.z + S[4 * i + 3] * q4.w;
           }
-          for (int off = CW; off < 64; off <<= 1) acc += __shfl_xor(acc, off, 64);
+#pragma unroll
+          for (int off = 1; off < KS; off <<= 1) acc += __shfl_xor(acc, off, 64);
           o = acc * rq;
         } else {
           const float fa = sc[tt * 4], fb = sc[tt * 4 + 1], em = sc[tt * 4 + 2];
           const float bv = fb * vj;
           float acc = 0.f, nq = 0.f;
 #pragma unroll
-          for (int i = 0; i < R; ++i) {
-            S[i] = fa * S[i] + kk[i] * bv;
-            acc += S[i] * qq[i];
-            N[i] = fa * N[i] + fb * kk[i];
-            nq += N[i] * qq[i];
+          for (int i = 0; i < R / 4; ++i) {
+            const float4 k4 = kk[i], q4 = qq[i];
+            const float kx[4] = {k4.x, k4.y, k4.z, k4.w}, qx[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              S[4 * i + j] = fa * S[4 * i + j] + kx[j] * bv;
+              acc += S[4 * i + j] * qx[j];
+              N[4 * i + j] = fa * N[4 * i + j] + fb * kx[j];
+              nq += N[4 * i + j] * qx[j];
+            }
           }
-          for (int off = CW; off < 64; off <<= 1) {
+#pragma unroll
+          for (int off = 1; off < KS; off <<= 1) {
             acc += __shfl_xor(acc, off, 64);
             nq += __shfl_xor(nq, off, 64);
           }
@@ -263,15 +334,27 @@ __global__ __launch_bounds__(256) void mlstm_commit_kernel(float* __restrict__ n
   for (int i = threadIdx.x; i < H; i += blockDim.x) mx[slot * H + i] = mx_new[(size_t)seq * H + i];
 }
 
-template <int MODE, typename TI>
-int launch_scan(const ScanArgs& a, int R, int n_seq, int nthreads, dim3 grid, hipStream_t st) {
-  const int NV = MODE == WKV ? 3 : 2;
-  const size_t lds = (size_t)(NV * TT * a.KS * (R + 4) + TT * a.CB + TT * 4) * sizeof(float);
+template <int MODE, typename TI, int R, int KS, int TT>
+int launch_scan_one(const ScanArgs& a, dim3 grid, hipStream_t st) {
+  constexpr int NV = MODE == WKV ? 3 : 2;
+  constexpr int KP = KS * (R + 4);
+  const size_t lds = (size_t)(NV * TT * KP + TT * a.CB + 8 * TT + (MODE == WKV ? KP : 0)) * sizeof(float);
   if (lds > 64 * 1024) return -6;
-  if (R == 16) linear_scan_kernel<MODE, TI, 16><<<grid, nthreads, lds, st>>>(a);
-  else if (R == 32) linear_scan_kernel<MODE, TI, 32><<<grid, nthreads, lds, st>>>(a);
-  else linear_scan_kernel<MODE, TI, 64><<<grid, nthreads, lds, st>>>(a);
+  linear_scan_kernel<MODE, TI, R, KS, TT><<<grid, 256, lds, st>>>(a);
   return 0;
+}
+
+template <int MODE, typename TI>
+int launch_scan(const ScanArgs& a, int R, dim3 grid, hipStream_t st) {
+  if (R == 32) return launch_scan_one<MODE, TI, 32, 16, 8>(a, grid, st);
+  switch (a.KS) {
+    case 1: return launch_scan_one<MODE, TI, 16, 1, 16>(a, grid, st);
+    case 2: return launch_scan_one<MODE, TI, 16, 2, 16>(a, grid, st);
+    case 4: return launch_scan_one<MODE, TI, 16, 4, 16>(a, grid, st);
+    case 8: return launch_scan_one<MODE, TI, 16, 8, 16>(a, grid, st);
+    case 16: return launch_scan_one<MODE, TI, 16, 16, 8>(a, grid, st);
+  }
+  return -5;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -375,11 +458,11 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   if (mode == MLSTM && (!norm || !mx || !aux2 || cap <= 0.f)) return -4;
   if (mode == WKV && (!par1 || !par2)) return -4;
   if (mode == DELTA && (!par1 || !par2 || !aux2)) return -4;
-  int R = r_sel > 0 ? r_sel : (dk <= 256 ? 16 : 32);
-  if (R != 16 && R != 32 && R != 64) return -5;
+  (void)r_sel;
+  const int R = dk <= 256 ? 16 : 32;               // key channels per thread; slices per column: a power of two up to 16
   int KS = 1;
   while (KS * R < dk) KS <<= 1;
-  if (KS > 64) return -5;
+  if (KS > 16) return -5;
   ScanArgs a;
   a.y = y; a.q = q; a.k = k; a.v = v;
   a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride;
@@ -391,9 +474,6 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   a.nwc = (dv + a.CW - 1) / a.CW;
   if (a.nwc > 4) a.nwc = 4;
   a.CB = a.nwc * a.CW;
-  const int lw = (KS * R + 63) / 64;
-  const int nthreads = 64 * (a.nwc > lw ? a.nwc : lw);
-  if (nthreads > 512) return -5;
   const int nz = (dv + a.CB - 1) / a.CB;
   if (H > 65535 || nz > 65535) return -5;
   const bool staged = mode == MLSTM && nz > 1;
@@ -403,7 +483,7 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   const dim3 grid(n_seq, H, nz);
   int rc;
 #define DGI_SCAN(M_)                                                                                      \
-  rc = in_f32 ? launch_scan<M_, float>(a, R, n_seq, nthreads, grid, st) : launch_scan<M_, uint16_t>(a, R, n_seq, nthreads, grid, st)
+  rc = in_f32 ? launch_scan<M_, float>(a, R, grid, st) : launch_scan<M_, uint16_t>(a, R, grid, st)
   if (mode == WKV) DGI_SCAN(WKV);
   else if (mode == DELTA) DGI_SCAN(DELTA);
   else DGI_SCAN(MLSTM);
@@ -419,10 +499,11 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
 
 // value columns one workgroup covers for this key size (the matrix memory stages its normaliser when dv exceeds it)
 extern "C" int dgi_linear_scan_columns(int dk, int dv, int r_sel) {
-  int R = r_sel > 0 ? r_sel : (dk <= 256 ? 16 : 32);
+  (void)r_sel;
+  const int R = dk <= 256 ? 16 : 32;
   int KS = 1;
   while (KS * R < dk) KS <<= 1;
-  if (KS > 64) return 0;
+  if (KS > 16) return 0;
   const int CW = 64 / KS;
   int nwc = (dv + CW - 1) / CW;
   if (nwc > 4) nwc = 4;
