@@ -767,7 +767,7 @@ void linear_scan(at::Tensor y, int64_t mode, const at::Tensor& q, const at::Tens
                            v.data_ptr(), (int)v.stride(0), f, aux1.data_ptr<float>(), (int)aux1.stride(0), a2, a2s,
                            f32p(par1, "par1", np), f32p(par2, "par2", np), state.data_ptr<float>(), nrm, mxp,
                            i32p(positions, "positions", T), i32p(seq_row0, "seq_row0", n_seq + 1),
-                           i32p(seq_slots, "seq_slots"), n_seq, (int)H, (int)G, (int)dk, (int)dv, (float)cap, (int)r_sel,
+                           i32p(seq_slots, "seq_slots"), n_seq, (int)H, (int)G, (int)dk, (int)dv, (float)cap, T,
                            nn, mn, cur_stream()), "linear_scan");
 }
 

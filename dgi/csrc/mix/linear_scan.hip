@@ -57,6 +57,30 @@ struct ScanArgs {
   float cap;
 };
 
+// Sums inside the vector ALU (data-parallel-primitive moves) instead of __shfl_xor, which goes through the LDS permute
+// unit: the sums sit on the token loop's dependent chain.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+// total over the KS adjacent lanes (aligned group, KS a power of two up to 16) that hold the slices of one column
+template <int KS>
+__device__ __forceinline__ float slice_sum(float v) {
+  if constexpr (KS >= 2) v += dpp_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  if constexpr (KS >= 4) v += dpp_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if constexpr (KS >= 8) v += dpp_move<0x141>(v);     // mirror inside each half row: the other quad's total
+  if constexpr (KS >= 16) v += dpp_move<0x140>(v);    // mirror inside the row: the other half's total
+  return v;
+}
+// total over a row of sixteen lanes, in every lane (four rotate-adds)
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<0x128>(v);
+  v += dpp_move<0x124>(v);
+  v += dpp_move<0x122>(v);
+  v += dpp_move<0x121>(v);
+  return v;
+}
+
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 __device__ __forceinline__ float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
@@ -208,11 +232,8 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
             r2 += qv * qv;
           }
         }
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) {
-          r1 += __shfl_xor(r1, off, 64);
-          if (MODE == DELTA) r2 += __shfl_xor(r2, off, 64);
-        }
+        r1 = row16_sum(r1);
+        if (MODE == DELTA) r2 = row16_sum(r2);
         if (l == 0) {
           if (MODE == WKV) {
             sc[tt * 4] = r1;
@@ -229,7 +250,8 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
     __syncthreads();
     if (t0 + TT < n) load_tile(t0 + TT);             // in flight while this tile is computed
     if (computes) {
-      for (int tt = 0; tt < nt; ++tt) {
+      // four tokens per trip: the LDS reads of the next tokens are issued under the arithmetic of the current one
+      auto token = [&](int tt) {
         const float4* kk = reinterpret_cast<const float4*>(sk + tt * KP + s * RP);
         const float4* qq = reinterpret_cast<const float4*>(sq + tt * KP + s * RP);
         const float vj = sv[tt * CB + cl];
@@ -246,8 +268,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
             S[4 * i + 2] = w4.z * S[4 * i + 2] + k4.z * vj;
             S[4 * i + 3] = w4.w * S[4 * i + 3] + k4.w * vj;
           }
-#pragma unroll
-          for (int off = 1; off < KS; off <<= 1) acc += __shfl_xor(acc, off, 64);
+          acc = slice_sum<KS>(acc);
           o = acc + sc[tt * 4] * vj;
         } else if constexpr (MODE == DELTA) {
           const float g = sc[tt * 4], beta = sc[tt * 4 + 1], rk = sc[tt * 4 + 2], rq = sc[tt * 4 + 3];
@@ -257,8 +278,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
             const float4 k4 = kk[i];
             pred += S[4 * i] * k4.x + S[4 * i + 1] * k4.y + S[4 * i + 2] * k4.z + S[4 * i + 3] * k4.w;
           }
-#pragma unroll
-          for (int off = 1; off < KS; off <<= 1) pred += __shfl_xor(pred, off, 64);
+          pred = slice_sum<KS>(pred);
           const float ku = beta * (vj - pred * g * rk) * rk;
           float acc = 0.f;
 #pragma unroll
@@ -270,8 +290,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
             S[4 * i + 3] = g * S[4 * i + 3] + k4.w * ku;
             acc += S[4 * i] * q4.x + S[4 * i + 1] * q4.y + S[4 * i + 2] * q4.z + S[4 * i + 3] * q4.w;
           }
-#pragma unroll
-          for (int off = 1; off < KS; off <<= 1) acc += __shfl_xor(acc, off, 64);
+          acc = slice_sum<KS>(acc);
           o = acc * rq;
         } else {
           const float fa = sc[tt * 4], fb = sc[tt * 4 + 1], em = sc[tt * 4 + 2];
@@ -289,15 +308,20 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
               nq += N[4 * i + j] * qx[j];
             }
           }
-#pragma unroll
-          for (int off = 1; off < KS; off <<= 1) {
-            acc += __shfl_xor(acc, off, 64);
-            nq += __shfl_xor(nq, off, 64);
-          }
+          acc = slice_sum<KS>(acc);
+          nq = slice_sum<KS>(nq);
           o = acc * qscale / (fmaxf(fabsf(nq * qscale), em) + 1e-6f);
         }
         if (s == 0 && col_ok) a.y[(size_t)(row0 + t0 + tt) * H * dv + (size_t)head * dv + col] = o;
+      };
+      int tt = 0;
+      for (; tt + 4 <= nt; tt += 4) {
+        token(tt);
+        token(tt + 1);
+        token(tt + 2);
+        token(tt + 3);
       }
+      for (; tt < nt; ++tt) token(tt);
     }
     __syncthreads();                                 // the tile is consumed before the next one overwrites it
   }
@@ -344,16 +368,20 @@ int launch_scan_one(const ScanArgs& a, dim3 grid, hipStream_t st) {
   return 0;
 }
 
+// short: a step of (nearly) single rows per sequence, i.e. decode: tiles of 4 tokens keep the staging registers few, so
+// more workgroups fit a compute unit and the step streams the states at a higher rate; prompt portions take 16-token tiles
 template <int MODE, typename TI>
-int launch_scan(const ScanArgs& a, int R, dim3 grid, hipStream_t st) {
-  if (R == 32) return launch_scan_one<MODE, TI, 32, 16, 8>(a, grid, st);
+int launch_scan(const ScanArgs& a, int R, bool short_rows, dim3 grid, hipStream_t st) {
+  if (R == 32) return short_rows ? launch_scan_one<MODE, TI, 32, 16, 4>(a, grid, st) : launch_scan_one<MODE, TI, 32, 16, 8>(a, grid, st);
+#define DGI_KS(K_, T_) return short_rows ? launch_scan_one<MODE, TI, 16, K_, 4>(a, grid, st) : launch_scan_one<MODE, TI, 16, K_, T_>(a, grid, st)
   switch (a.KS) {
-    case 1: return launch_scan_one<MODE, TI, 16, 1, 16>(a, grid, st);
-    case 2: return launch_scan_one<MODE, TI, 16, 2, 16>(a, grid, st);
-    case 4: return launch_scan_one<MODE, TI, 16, 4, 16>(a, grid, st);
-    case 8: return launch_scan_one<MODE, TI, 16, 8, 16>(a, grid, st);
-    case 16: return launch_scan_one<MODE, TI, 16, 16, 8>(a, grid, st);
+    case 1: DGI_KS(1, 16);
+    case 2: DGI_KS(2, 16);
+    case 4: DGI_KS(4, 16);
+    case 8: DGI_KS(8, 16);
+    case 16: DGI_KS(16, 8);
   }
+#undef DGI_KS
   return -5;
 }
 
@@ -415,6 +443,69 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(TO* __restrict__ ou
   }
 }
 
+
+template <typename T> __device__ __forceinline__ void ld4v(const T* p, float* f);
+template <> __device__ __forceinline__ void ld4v<uint16_t>(const uint16_t* p, float* f) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void ld4v<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <typename T> __device__ __forceinline__ void st4v(T* p, const float* f);
+template <> __device__ __forceinline__ void st4v<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ void st4v<uint16_t>(uint16_t* p, const float* f) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]));
+}
+
+// Sixteen lanes per (row, head), four columns per access (dv a multiple of 4, at most 256): the head's values stay in
+// registers between the sum of squares (four rotate-adds inside the row of lanes) and the store.
+template <typename TZ, typename TO>
+__global__ __launch_bounds__(256) void head_norm_gate_vec_kernel(TO* __restrict__ out, const float* __restrict__ y,
+                                                                 const TZ* __restrict__ z, int z_stride,
+                                                                 const float* __restrict__ w, int wlen, int T, int H, int dv,
+                                                                 float eps, int sigmoid_gate) {
+  constexpr int MAXCH = 4;
+  const long long unit = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = unit < (long long)T * H;
+  const int t = live ? (int)(unit / H) : 0, head = live ? (int)(unit - (long long)t * H) : 0;
+  const int l = threadIdx.x & 15;
+  const float* yp = y + ((size_t)t * H + head) * dv;
+  float v[MAXCH][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < MAXCH; ++k) {
+    const int c = (l + 16 * k) * 4;
+    if (live && c < dv) {
+      ld4v<float>(yp + c, v[k]);
+      ss += v[k][0] * v[k][0] + v[k][1] * v[k][1] + v[k][2] * v[k][2] + v[k][3] * v[k][3];
+    }
+  }
+  const float inv = 1.f / sqrtf(row16_sum(ss) / (float)dv + eps);
+  if (!live) return;
+  const TZ* zp = z + (size_t)t * z_stride + (size_t)head * dv;
+  TO* op = out + ((size_t)t * H + head) * dv;
+#pragma unroll
+  for (int k = 0; k < MAXCH; ++k) {
+    const int c = (l + 16 * k) * 4;
+    if (c < dv) {
+      float g[4], wv[4], o[4];
+      ld4v<TZ>(zp + c, g);
+      ld4v<float>(w + (head * dv + c) % wlen, wv);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float sg = 1.f / (1.f + expf(-g[j]));
+        o[j] = v[k][j] * inv * wv[j] * (sigmoid_gate ? sg : g[j] * sg);
+      }
+      st4v<TO>(op + c, o);
+    }
+  }
+}
+
 template <typename TA>
 __global__ __launch_bounds__(256) void rms_pair_mean_kernel(float* __restrict__ out, const TA* __restrict__ a, int a_stride,
                                                             const TA* __restrict__ b, int b_stride,
@@ -445,20 +536,19 @@ __global__ __launch_bounds__(256) void rms_pair_mean_kernel(float* __restrict__ 
 
 }  // namespace
 
-// mode 0 wkv, 1 delta, 2 mlstm; q / k / v bf16 or fp32 (in_f32) with row strides in elements.
-// r_sel > 0 forces the key channels per thread (16 / 32 / 64), 0 picks them from dk.
+// mode 0 wkv, 1 delta, 2 mlstm; q / k / v bf16 or fp32 (in_f32) with row strides in elements; rows: rows of the step.
 extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, const void* k, int k_stride, const void* v,
                                int v_stride, int in_f32, const float* aux1, int aux1_stride, const float* aux2,
                                int aux2_stride, const float* par1, const float* par2, float* state, float* norm, float* mx,
                                const int* positions, const int* seq_row0, const int* seq_slots, int n_seq, int H, int G,
-                               int dk, int dv, float cap, int r_sel, float* norm_new, float* mx_new, hipStream_t st) {
+                               int dk, int dv, float cap, int rows, float* norm_new, float* mx_new, hipStream_t st) {
   if (n_seq == 0) return 0;
   if (mode < 0 || mode > 2 || H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0) return -2;
   if (dk > 512) return -3;
   if (mode == MLSTM && (!norm || !mx || !aux2 || cap <= 0.f)) return -4;
   if (mode == WKV && (!par1 || !par2)) return -4;
   if (mode == DELTA && (!par1 || !par2 || !aux2)) return -4;
-  (void)r_sel;
+  const bool short_rows = rows <= 4 * n_seq;       // rows of the step: at most four per sequence on average
   const int R = dk <= 256 ? 16 : 32;               // key channels per thread; slices per column: a power of two up to 16
   int KS = 1;
   while (KS * R < dk) KS <<= 1;
@@ -483,7 +573,7 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   const dim3 grid(n_seq, H, nz);
   int rc;
 #define DGI_SCAN(M_)                                                                                      \
-  rc = in_f32 ? launch_scan<M_, float>(a, R, grid, st) : launch_scan<M_, uint16_t>(a, R, grid, st)
+  rc = in_f32 ? launch_scan<M_, float>(a, R, short_rows, grid, st) : launch_scan<M_, uint16_t>(a, R, short_rows, grid, st)
   if (mode == WKV) DGI_SCAN(WKV);
   else if (mode == DELTA) DGI_SCAN(DELTA);
   else DGI_SCAN(MLSTM);
@@ -533,10 +623,17 @@ extern "C" int dgi_head_norm_gate(void* out, int out_f32, const float* y, const 
   if (T == 0) return 0;
   if (H <= 0 || dv <= 0 || wlen <= 0 || (H * dv) % wlen) return -2;
   const long long units = (long long)T * H;
-  const unsigned blocks = (unsigned)((units + 3) / 4);
+  // 16-byte path: head sizes, weight period, row strides and pointers in fours
+  const bool vec = dv % 4 == 0 && dv <= 256 && wlen % 4 == 0 && z_stride % 4 == 0 &&
+                   (((uintptr_t)out | (uintptr_t)y | (uintptr_t)z | (uintptr_t)w) & 15) == 0;
+  const unsigned blocks = (unsigned)(vec ? (units + 15) / 16 : (units + 3) / 4);
 #define DGI_HNG(TZ_, TO_)                                                                                             \
-  head_norm_gate_kernel<TZ_, TO_><<<blocks, 256, 0, st>>>((TO_*)out, y, (const TZ_*)z, z_stride, w, wlen, T, H, dv, eps, \
-                                                          sigmoid_gate)
+  do {                                                                                                                \
+    if (vec) head_norm_gate_vec_kernel<TZ_, TO_><<<blocks, 256, 0, st>>>((TO_*)out, y, (const TZ_*)z, z_stride, w, wlen, T, H, \
+                                                                        dv, eps, sigmoid_gate);                       \
+    else head_norm_gate_kernel<TZ_, TO_><<<blocks, 256, 0, st>>>((TO_*)out, y, (const TZ_*)z, z_stride, w, wlen, T, H, dv, eps, \
+                                                                sigmoid_gate);                                        \
+  } while (0)
   if (z_f32) { if (out_f32) DGI_HNG(float, float); else DGI_HNG(float, uint16_t); }
   else { if (out_f32) DGI_HNG(uint16_t, float); else DGI_HNG(uint16_t, uint16_t); }
 #undef DGI_HNG
