@@ -3,7 +3,8 @@
 // clamped GLU and soft-capped logits.  A library of its own, so a model that needs only these
 // builds in seconds; it registers into the same `dgi` namespace as dgi/_C.so (as a fragment).
 // Shapes are checked here, on the host, before any launch; every op runs on the current stream
-// and allocates nothing.
+// and allocates nothing (one exception: a matrix-memory scan whose heads span several workgroups
+// stages two small rows per sequence, from the caching allocator).
 #include <torch/library.h>
 #include <ATen/ATen.h>
 #include <c10/hip/HIPStream.h>
@@ -62,8 +63,8 @@ int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, const void*
                     int v_stride, int in_f32, const float* aux1, int aux1_stride, const float* aux2, int aux2_stride,
                     const float* par1, const float* par2, float* state, float* norm, float* mx, const int* positions,
                     const int* seq_row0, const int* seq_slots, int n_seq, int H, int G, int dk, int dv, float cap,
-                    int r_sel, float* norm_new, float* mx_new, hipStream_t st);
-int dgi_linear_scan_columns(int dk, int dv, int r_sel);
+                    int rows, float* norm_new, float* mx_new, hipStream_t st);
+int dgi_linear_scan_columns(int dk, int dv);
 int dgi_token_shift(void* out, int out_f32, const void* h, int h_f32, int h_stride, const float* mu, int nmix, float* tail,
                     const int* positions, const int* row_seq, const int* seq_row0, const int* seq_slots, int n_seq, int T,
                     int W, hipStream_t st);
@@ -724,7 +725,7 @@ void linear_scan(at::Tensor y, int64_t mode, const at::Tensor& q, const at::Tens
                  const at::Tensor& aux1, const c10::optional<at::Tensor>& aux2, const c10::optional<at::Tensor>& par1,
                  const c10::optional<at::Tensor>& par2, at::Tensor state, c10::optional<at::Tensor> norm,
                  c10::optional<at::Tensor> mx, const at::Tensor& positions, const at::Tensor& seq_row0,
-                 const at::Tensor& seq_slots, int64_t H, int64_t G, int64_t dk, int64_t dv, double cap, int64_t r_sel) {
+                 const at::Tensor& seq_slots, int64_t H, int64_t G, int64_t dk, int64_t dv, double cap) {
   check_f32(y, "y"); check_f32(state, "state");
   const int f = act_kind(q, "q");
   TORCH_CHECK(act_kind(k, "k") == f && act_kind(v, "v") == f, "linear_scan: q, k, v must share a dtype");
@@ -758,7 +759,7 @@ void linear_scan(at::Tensor y, int64_t mode, const at::Tensor& q, const at::Tens
   // a matrix memory whose heads span several column blocks stages its new normaliser / maximum (committed by a second launch)
   at::Tensor norm_new, mx_new;
   float *nn = nullptr, *mn = nullptr;
-  if (mode == 2 && n_seq > 0 && dgi_linear_scan_columns((int)dk, (int)dv, (int)r_sel) < dv) {
+  if (mode == 2 && n_seq > 0 && dgi_linear_scan_columns((int)dk, (int)dv) < dv) {
     norm_new = at::empty({n_seq, H, dk}, state.options());
     mx_new = at::empty({n_seq, H}, state.options());
     nn = norm_new.data_ptr<float>(); mn = mx_new.data_ptr<float>();
@@ -855,7 +856,7 @@ TORCH_LIBRARY_FRAGMENT(dgi, m) {
         "int qt_every=0) -> ()");
   m.def("linear_scan(Tensor(a!) y, int mode, Tensor q, Tensor k, Tensor v, Tensor aux1, Tensor? aux2, Tensor? par1, Tensor? par2, "
         "Tensor(b!) state, Tensor(c!)? norm, Tensor(d!)? mx, Tensor positions, Tensor seq_row0, Tensor seq_slots, int H, int G, "
-        "int dk, int dv, float cap, int r_sel=0) -> ()");
+        "int dk, int dv, float cap) -> ()");
   m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) tail, Tensor positions, Tensor row_seq, Tensor seq_row0, "
         "Tensor seq_slots) -> ()");
   m.def("head_norm_gate(Tensor(a!) out, Tensor y, Tensor z, Tensor w, int heads, float eps, int sigmoid_gate) -> ()");

@@ -588,8 +588,7 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
 }
 
 // value columns one workgroup covers for this key size (the matrix memory stages its normaliser when dv exceeds it)
-extern "C" int dgi_linear_scan_columns(int dk, int dv, int r_sel) {
-  (void)r_sel;
+extern "C" int dgi_linear_scan_columns(int dk, int dv) {
   const int R = dk <= 256 ? 16 : 32;
   int KS = 1;
   while (KS * R < dk) KS <<= 1;
