@@ -293,7 +293,9 @@ class LofuvikModel:
         T = h.shape[0]
         xs = linrec.token_shift(h, L.mu, st[f"shift.{r}"], meta.positions, meta.row_seq, meta.seq_row0, meta.seq_slots,
                                 self.dtype)                                             # [5, T, W]
-        rkvg = torch.bmm(xs[:4], L.rkvg.transpose(1, 2))                                # [4, T, H*D]
+        # one plain GEMM per blend (a skinny-row kernel at decode sizes): the vendor's batched bf16 product of these
+        # four faulted at 32 rows x 2048 x 2048, so no batched call here
+        rkvg = [ops.linear(xs[i], L.rkvg[i]) for i in range(4)]                         # 4 x [T, H*D]
         low = torch.tanh(torch.nn.functional.linear(xs[4].float(), L.w1))
         w_raw = torch.nn.functional.linear(low, L.w2)                                   # fp32 decay logits
         y = linrec.wkv_scan(rkvg[0], rkvg[1], rkvg[2], w_raw, L.w0, L.bonus, st[f"mem.{r}"], meta.positions,
