@@ -64,7 +64,7 @@ int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, const void*
                     const float* par1, const float* par2, float* state, float* norm, float* mx, const int* positions,
                     const int* seq_row0, const int* seq_slots, int n_seq, int H, int G, int dk, int dv, float cap,
                     int rows, float* norm_new, float* mx_new, hipStream_t st);
-int dgi_linear_scan_columns(int dk, int dv);
+int dgi_linear_scan_columns(int dk, int dv, int H, int n_seq, int rows);
 int dgi_token_shift(void* out, int out_f32, const void* h, int h_f32, int h_stride, const float* mu, int nmix, float* tail,
                     const int* positions, const int* row_seq, const int* seq_row0, const int* seq_slots, int n_seq, int T,
                     int W, hipStream_t st);
@@ -759,7 +759,7 @@ void linear_scan(at::Tensor y, int64_t mode, const at::Tensor& q, const at::Tens
   // a matrix memory whose heads span several column blocks stages its new normaliser / maximum (committed by a second launch)
   at::Tensor norm_new, mx_new;
   float *nn = nullptr, *mn = nullptr;
-  if (mode == 2 && n_seq > 0 && dgi_linear_scan_columns((int)dk, (int)dv) < dv) {
+  if (mode == 2 && n_seq > 0 && dgi_linear_scan_columns((int)dk, (int)dv, (int)H, n_seq, T) < dv) {
     norm_new = at::empty({n_seq, H, dk}, state.options());
     mx_new = at::empty({n_seq, H}, state.options());
     nn = norm_new.data_ptr<float>(); mn = mx_new.data_ptr<float>();

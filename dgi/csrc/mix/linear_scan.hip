@@ -373,6 +373,10 @@ int launch_scan_one(const ScanArgs& a, dim3 grid, hipStream_t st) {
 template <int MODE, typename TI>
 int launch_scan(const ScanArgs& a, int R, bool short_rows, dim3 grid, hipStream_t st) {
   if (R == 32) return short_rows ? launch_scan_one<MODE, TI, 32, 16, 4>(a, grid, st) : launch_scan_one<MODE, TI, 32, 16, 8>(a, grid, st);
+  if (R == 4 && a.KS == 16) return launch_scan_one<MODE, TI, 4, 16, 16>(a, grid, st);
+  if (R == 8 && a.KS == 8) return launch_scan_one<MODE, TI, 8, 8, 16>(a, grid, st);
+  if (R == 8 && a.KS == 16) return launch_scan_one<MODE, TI, 8, 16, 16>(a, grid, st);
+  if (R != 16) return -5;
 #define DGI_KS(K_, T_) return short_rows ? launch_scan_one<MODE, TI, 16, K_, 4>(a, grid, st) : launch_scan_one<MODE, TI, 16, K_, T_>(a, grid, st)
   switch (a.KS) {
     case 1: DGI_KS(1, 16);
@@ -536,6 +540,38 @@ __global__ __launch_bounds__(256) void rms_pair_mean_kernel(float* __restrict__ 
 
 }  // namespace
 
+// value columns of one workgroup with KS lanes per column: up to four waves of 64 / KS columns
+static int scan_columns(int KS, int dv) {
+  const int CW = 64 / KS;
+  int nwc = (dv + CW - 1) / CW;
+  if (nwc > 4) nwc = 4;
+  return nwc * CW;
+}
+
+// Key channels per thread.  A decode-shaped step streams the states: 16 channels per thread, all columns of a head in
+// one workgroup.  A prompt portion is a dependent chain per (sequence, head, column) whose length per token grows with
+// the channels a thread holds, so while the grid stays within two workgroups per compute unit a head is spread over
+// more lanes per column (and so over more workgroups): 4 or 8 channels per thread.  Beyond that the step is bound by
+// the instructions issued, and the wide layout issues the fewest.
+static int scan_channels(int dk, int dv, int H, int n_seq, int rows) {
+  if (dk > 256) return 32;
+  if (rows <= 4 * n_seq) return 16;
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    return n > 0 ? n : 256;
+  }();
+  for (int R = 4; R <= 8; R *= 2) {
+    int KS = 1;
+    while (KS * R < dk) KS <<= 1;
+    if (!((R == 4 && KS == 16) || (R == 8 && (KS == 8 || KS == 16)))) continue;      // the layouts instantiated
+    const int CB = scan_columns(KS, dv);
+    const long grid = (long)n_seq * H * ((dv + CB - 1) / CB);
+    if (grid <= 2L * cus) return R;
+  }
+  return 16;
+}
+
 // mode 0 wkv, 1 delta, 2 mlstm; q / k / v bf16 or fp32 (in_f32) with row strides in elements; rows: rows of the step.
 extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, const void* k, int k_stride, const void* v,
                                int v_stride, int in_f32, const float* aux1, int aux1_stride, const float* aux2,
@@ -549,7 +585,7 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   if (mode == WKV && (!par1 || !par2)) return -4;
   if (mode == DELTA && (!par1 || !par2 || !aux2)) return -4;
   const bool short_rows = rows <= 4 * n_seq;       // rows of the step: at most four per sequence on average
-  const int R = dk <= 256 ? 16 : 32;               // key channels per thread; slices per column: a power of two up to 16
+  const int R = scan_channels(dk, dv, H, n_seq, rows);
   int KS = 1;
   while (KS * R < dk) KS <<= 1;
   if (KS > 16) return -5;
@@ -561,9 +597,8 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   a.positions = positions; a.seq_row0 = seq_row0; a.seq_slots = seq_slots;
   a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.cap = cap;
   a.KS = KS; a.CW = 64 / KS;
-  a.nwc = (dv + a.CW - 1) / a.CW;
-  if (a.nwc > 4) a.nwc = 4;
-  a.CB = a.nwc * a.CW;
+  a.CB = scan_columns(KS, dv);
+  a.nwc = a.CB / a.CW;
   const int nz = (dv + a.CB - 1) / a.CB;
   if (H > 65535 || nz > 65535) return -5;
   const bool staged = mode == MLSTM && nz > 1;
@@ -587,16 +622,13 @@ extern "C" int dgi_linear_scan(float* y, int mode, const void* q, int q_stride, 
   return 0;
 }
 
-// value columns one workgroup covers for this key size (the matrix memory stages its normaliser when dv exceeds it)
-extern "C" int dgi_linear_scan_columns(int dk, int dv) {
-  const int R = dk <= 256 ? 16 : 32;
+// value columns one workgroup covers in this step (the matrix memory stages its normaliser when dv exceeds it)
+extern "C" int dgi_linear_scan_columns(int dk, int dv, int H, int n_seq, int rows) {
+  const int R = scan_channels(dk, dv, H, n_seq, rows);
   int KS = 1;
   while (KS * R < dk) KS <<= 1;
   if (KS > 16) return 0;
-  const int CW = 64 / KS;
-  int nwc = (dv + CW - 1) / CW;
-  if (nwc > 4) nwc = 4;
-  return nwc * CW;
+  return scan_columns(KS, dv);
 }
 
 extern "C" int dgi_token_shift(void* out, int out_f32, const void* h, int h_f32, int h_stride, const float* mu, int nmix,

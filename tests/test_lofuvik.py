@@ -285,7 +285,34 @@ def scan_params(g, mode, H, D):
 
 SCAN_GEOMS = [("wkv", 2, 2, 12, 12), ("wkv", 3, 3, 64, 64), ("wkv", 1, 1, 5, 5), ("wkv", 2, 2, 130, 130),
               ("delta", 4, 2, 6, 10), ("delta", 3, 3, 20, 4), ("delta", 2, 1, 128, 64), ("delta", 6, 2, 16, 70),
-              ("mlstm", 2, 2, 10, 6), ("mlstm", 3, 3, 4, 20), ("mlstm", 2, 2, 64, 128), ("mlstm", 1, 1, 300, 17)]
+              ("mlstm", 2, 2, 10, 6), ("mlstm", 3, 3, 4, 20), ("mlstm", 2, 2, 64, 128), ("mlstm", 1, 1, 300, 17),
+              ("delta", 2, 1, 48, 40), ("mlstm", 2, 2, 100, 33), ("wkv", 2, 2, 40, 40)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads", [6, 48, 64])
+@pytest.mark.parametrize("mode", ["wkv", "delta", "mlstm"])
+def test_recurrences_prompt_steps_of_every_grid_size(mode, heads):
+    """A prompt step picks its thread layout by the number of workgroups (sequences x heads x column blocks): five
+    sequences of nine rows with few, many and very many heads take the three layouts; each continues a state."""
+    H, G, D, V, n, ns = heads, heads // 2, 64, 64, 9, 5
+    g = torch.Generator().manual_seed(heads)
+    par = scan_params(g, mode, H, D)
+    st = {"S": torch.randn(ns + 1, H, D, V, generator=g) * 0.3, "n": torch.randn(ns + 1, H, D, generator=g) * 0.3,
+          "m": torch.randn(ns + 1, H, generator=g).abs()}
+    if mode != "delta":
+        G = H
+    ins = [scan_inputs(g, mode, H, G, D, V, n, torch.float32) for _ in range(ns)]
+    cat = [None if ins[0][j] is None else torch.cat([x[j] for x in ins], 0) for j in range(5)]
+    out = {}
+    for device in ("cpu", "cuda"):
+        pos, rs, r0, sl = seq_meta([n] * ns, [3] * ns, list(range(1, ns + 1)), device)
+        sd = {k: v.clone().to(device) for k, v in st.items()}
+        y = scan_call(mode, *[None if c is None else c.to(device) for c in cat], par, sd, pos, r0, sl, H, G, D, V)
+        out[device] = [y.cpu()] + [sd[k].cpu() for k in ("S", "n", "m")]
+    for a, b in zip(out["cuda"], out["cpu"]):
+        scale = b.abs().max().clamp(min=1.0)
+        close(a / scale, b / scale, 2e-5)
 
 
 @pytest.mark.parametrize("device", DEVICES)
