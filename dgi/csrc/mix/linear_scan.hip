@@ -250,8 +250,9 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
     __syncthreads();
     if (t0 + TT < n) load_tile(t0 + TT);             // in flight while this tile is computed
     if (computes) {
-      // four tokens per trip: the LDS reads of the next tokens are issued under the arithmetic of the current one
-      auto token = [&](int tt) {
+      // four tokens per trip, free of branches (the outputs wait in registers and are stored after the trip), so the
+      // LDS reads of the later tokens are issued under the arithmetic of the earlier ones
+      auto token = [&](int tt) -> float {
         const float4* kk = reinterpret_cast<const float4*>(sk + tt * KP + s * RP);
         const float4* qq = reinterpret_cast<const float4*>(sq + tt * KP + s * RP);
         const float vj = sv[tt * CB + cl];
@@ -312,16 +313,24 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
           nq = slice_sum<KS>(nq);
           o = acc * qscale / (fmaxf(fabsf(nq * qscale), em) + 1e-6f);
         }
-        if (s == 0 && col_ok) a.y[(size_t)(row0 + t0 + tt) * H * dv + (size_t)head * dv + col] = o;
+        return o;
       };
+      const size_t ys = (size_t)H * dv;
+      float* yp = a.y + (size_t)(row0 + t0) * ys + (size_t)head * dv + col;
       int tt = 0;
       for (; tt + 4 <= nt; tt += 4) {
-        token(tt);
-        token(tt + 1);
-        token(tt + 2);
-        token(tt + 3);
+        const float o0 = token(tt), o1 = token(tt + 1), o2 = token(tt + 2), o3 = token(tt + 3);
+        if (s == 0 && col_ok) {
+          yp[tt * ys] = o0;
+          yp[(tt + 1) * ys] = o1;
+          yp[(tt + 2) * ys] = o2;
+          yp[(tt + 3) * ys] = o3;
+        }
       }
-      for (; tt < nt; ++tt) token(tt);
+      for (; tt < nt; ++tt) {
+        const float o = token(tt);
+        if (s == 0 && col_ok) yp[tt * ys] = o;
+      }
     }
     __syncthreads();                                 // the tile is consumed before the next one overwrites it
   }
